@@ -1,0 +1,187 @@
+/*
+ * moe_a2a.h — C ABI of the MI355X (gfx950) MoE dispatch/combine library.
+ *
+ * One rank's share of the single-node MoE all-to-all of the reference's
+ * `all2all` task: count -> stable order -> pack -> [exchange] -> expert-major
+ * placement -> [expert] -> gather -> [exchange] -> weighted combine.
+ *
+ * Conventions shared by every entry point
+ *   - all pointers are DEVICE pointers unless a parameter says "host";
+ *   - token rows are 2-byte elements (fp16 or bf16), `hidden_dim` of them,
+ *     contiguous, rows back to back; meta rows are 5 x int32
+ *     {global_expert, src_rank, src_token, src_k, pad}
+ *     (reference: all2all/reference.py:56 `META_DIM = 5`);
+ *   - nothing is allocated, freed or cleared by the library; every output
+ *     buffer is owned by the caller; no entry point synchronises the host;
+ *   - `stream` is a hipStream_t passed as void*; NULL is the null stream;
+ *   - every `rows_hint` is a host-side upper-bound guess of the number of
+ *     rows the call will move. It only sizes the launch: kernels read the
+ *     true row count from device memory and stride over it, so a wrong hint
+ *     costs time, never correctness;
+ *   - return value: MOE_A2A_OK (0) or a negative MOE_A2A_E* code. Argument
+ *     errors are detected before anything is launched.
+ *
+ * Ordering contract (what makes results identical to the reference): every
+ * permutation below is a STABLE partition of its input stream, computed by
+ * ranking (no atomics), so slots do not depend on scheduling.
+ */
+#ifndef MOE_A2A_H_
+#define MOE_A2A_H_
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MOE_A2A_META_DIM 5
+
+/* element types of token rows (reference: MoEConfig.in_dtype / out_dtype,
+ * all2all/reference.py:16-17) */
+#define MOE_A2A_F16 0
+#define MOE_A2A_BF16 1
+
+#define MOE_A2A_OK 0
+#define MOE_A2A_EINVAL (-1)   /* bad size / null pointer / unsupported value */
+#define MOE_A2A_EALIGN (-2)   /* a row buffer is not 2-byte aligned */
+#define MOE_A2A_ELAUNCH (-3)  /* hipGetLastError() != hipSuccess after launch */
+
+/* Static shape of one rank's problem (reference: MoEConfig,
+ * all2all/reference.py:10-17, and PyTorchAllToAll.__init__, :58-65). */
+typedef struct moe_a2a_shape {
+  int32_t world_size;        /* W; num_local_experts = num_experts / W     */
+  int32_t rank;              /* this rank, 0 <= rank < W                    */
+  int32_t num_experts;       /* E, multiple of W, <= 65536                  */
+  int32_t experts_per_token; /* K                                           */
+  int32_t hidden_dim;        /* H elements per token row                    */
+  int32_t max_num_tokens;    /* per-rank token capacity; max_recv = this*W  */
+} moe_a2a_shape;
+
+/* Library version / build probe. Returns a static string such as
+ * "moe_a2a 0.1 gfx950". Never NULL. */
+const char* moe_a2a_version(void);
+
+/* Human-readable text for a status code. Never NULL. */
+const char* moe_a2a_strerror(int status);
+
+/*
+ * Dispatch, send side.
+ * Replaces all2all/reference.py:74-86,93,100-102 (loop over indices building
+ * send_counts / token_map / meta_map, then the per-destination row gather).
+ *
+ *   x           [num_tokens, H]  token rows
+ *   indices     [num_tokens, K]  int32 global expert ids
+ *   send_buf    [num_tokens*K, H] out: rows grouped by destination rank
+ *                                (rank 0 first), inside a group in (t, k)
+ *                                order — a stable sort of the t-major,
+ *                                k-minor stream by indices[t,k] / nle
+ *   send_meta   [num_tokens*K, 5] out: {e, rank, t, k, 0} per sent row
+ *   send_counts [W] int32        out: rows per destination rank
+ *   send_slot   [num_tokens*K]   out, optional (may be NULL): row of
+ *                                send_buf that entry t*K+k went to
+ */
+int moe_a2a_dispatch_send(const moe_a2a_shape* shape, const void* x,
+                          const int32_t* indices, int32_t num_tokens,
+                          void* send_buf, int32_t* send_meta,
+                          int32_t* send_counts, int32_t* send_slot,
+                          void* stream);
+
+/*
+ * Dispatch, receive side: received stream -> expert-major buffers.
+ * Replaces all2all/reference.py:123-146 (per received row:
+ * le = meta[0] % nle; expert_x[le, cnt[le]++] = row).
+ *
+ *   recv_buf    [R, H]  rows as the exchange delivered them: source rank 0's
+ *                       segment first, each in the sender's order
+ *   recv_meta   [R, 5]
+ *   recv_counts [W] int32, rows received from each source rank; R = their sum
+ *   expert_num_tokens [nle] int32 out (every entry written, zeros included)
+ *   expert_x    [nle, max_recv, H] out; only rows < expert_num_tokens[le] are
+ *                       written (the reference leaves the rest uninitialised
+ *                       too: torch.empty at reference.py:127)
+ *   expert_meta [nle, max_recv, 5] out, same rule
+ * A row whose position inside its expert would reach max_recv is not stored;
+ * expert_num_tokens still counts it, so overflow is visible to the caller.
+ */
+int moe_a2a_dispatch_recv(const moe_a2a_shape* shape, const void* recv_buf,
+                          const int32_t* recv_meta, const int32_t* recv_counts,
+                          int32_t rows_hint, int32_t* expert_num_tokens,
+                          void* expert_x, int32_t* expert_meta, void* stream);
+
+/*
+ * Combine, send side: expert-major results -> rows grouped by origin rank.
+ * Replaces all2all/reference.py:163-199 (loop le ascending, j < cnt[le]
+ * ascending, bucket by meta[1]; concatenate buckets in rank order).
+ *
+ *   expert_y    [nle, max_recv, H], expert_meta [nle, max_recv, 5],
+ *   expert_num_tokens [nle] (values above max_recv are clamped)
+ *   send_buf    [R, H] out, send_meta [R, 5] out (meta rows copied unchanged)
+ *   send_counts [W] int32 out
+ */
+int moe_a2a_combine_send(const moe_a2a_shape* shape, const void* expert_y,
+                         const int32_t* expert_meta,
+                         const int32_t* expert_num_tokens, int32_t rows_hint,
+                         void* send_buf, int32_t* send_meta,
+                         int32_t* send_counts, void* stream);
+
+/*
+ * Combine, receive side: weighted sum back into token order.
+ * Replaces all2all/reference.py:227-232
+ *   out_tokens[src_token] += recv_buf[i].to(float32) * weights[src_token, src_k]
+ * for i in arrival order. out_tokens has the 16-bit element type, so the
+ * running sum is rounded to it after EVERY addend:
+ *   p = RN32(f32(v) * w);  a = RN32(f32(acc) + p);  acc = RN16(a)
+ * (separate multiply and add, no fma). The kernel reproduces exactly that.
+ *
+ *   recv_buf    [R, H], recv_meta [R, 5], recv_counts [W] int32 (R = sum)
+ *   weights     [num_tokens, K] float32
+ *   out_tokens  [num_tokens, H] in/out
+ *   accumulate  nonzero: start from the values already in out_tokens (the
+ *               reference's in-place +=); zero: start from +0 and overwrite,
+ *               which equals the reference on its zero-initialised buffer
+ *               (reference.py:263-268) without reading it
+ *   dtype       MOE_A2A_F16 or MOE_A2A_BF16: element type of recv_buf and
+ *               out_tokens
+ * Rows whose src_token or src_k is out of range are ignored.
+ */
+int moe_a2a_combine_recv(const moe_a2a_shape* shape, const void* recv_buf,
+                         const int32_t* recv_meta, const int32_t* recv_counts,
+                         const float* weights, int32_t num_tokens,
+                         void* out_tokens, int32_t accumulate, int32_t dtype,
+                         void* stream);
+
+/*
+ * Stand-in for the expert computation between dispatch and combine.
+ * Replaces all2all/reference.py:262
+ *   expert_y = expert_x.to(out_dtype) * (1 + rank)
+ * on the valid rows only (j < expert_num_tokens[le]): per element
+ *   RN_out( f32( RN_out( f32(x) ) ) * float(1 + rank) ).
+ */
+int moe_a2a_expert_scale(const moe_a2a_shape* shape, const void* expert_x,
+                         const int32_t* expert_num_tokens, int32_t rows_hint,
+                         int32_t in_dtype, int32_t out_dtype, void* expert_y,
+                         void* stream);
+
+/*
+ * Stand-in for one (source rank -> destination rank) leg of the exchange,
+ * done as a device copy on one GPU. Replaces, for that leg, the three
+ * dist.all_to_all_single calls at all2all/reference.py:107-119 (dispatch)
+ * and :210-222 (combine).
+ *
+ * Copies the segment the source holds for `dst_rank` (rows
+ * [sum(send_counts[:dst_rank]), +send_counts[dst_rank])) of send_buf/send_meta
+ * to rows [sum(recv_counts[:src_rank]), ...) of recv_buf/recv_meta.
+ * send_counts belongs to the source rank, recv_counts to the destination;
+ * the copy moves min(send_counts[dst_rank], recv_counts[src_rank]) rows.
+ */
+int moe_a2a_exchange_local(int32_t world_size, int32_t hidden_dim,
+                           const void* send_buf, const int32_t* send_meta,
+                           const int32_t* send_counts, int32_t dst_rank,
+                           void* recv_buf, int32_t* recv_meta,
+                           const int32_t* recv_counts, int32_t src_rank,
+                           int32_t rows_hint, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MOE_A2A_H_ */
