@@ -1,0 +1,269 @@
+#!/usr/bin/env python3
+"""Benchmark of one rank's MoE dispatch+combine on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload C4] [--mode graph|eager]
+
+A step is one pass of rank 0's share of the job, everything on the device and
+on one stream:
+
+    dispatch_send -> [exchange leg 0->0] -> dispatch_recv -> [expert stand-in]
+      -> combine_send -> [exchange leg 0->0] -> combine_recv
+
+The bracketed launches are the stand-ins for what is outside this path (the
+xGMI exchange, the expert GEMM). The seven peers' inbound segments are produced
+once, before timing, by running the peers' own kernels on their seeded inputs;
+they stay resident where an exchange would have written them.
+
+Prints ONE JSON line. `value` is the wall time of a whole step (stand-ins
+included) in microseconds; `hot_path_us` is the sum of the four path kernels
+alone, each timed with HIP events on the launch stream; `roofline` prices the
+slowest of those four against HBM peak with the algorithmic bytes of that
+stage; `cpu_baseline` is the row-by-row torch-CPU statement of the same step
+timed on this box's host cores.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import statistics
+import sys
+import time
+from pathlib import Path
+
+ROOT = Path(__file__).resolve().parent
+if str(ROOT) not in sys.path:
+    sys.path.insert(0, str(ROOT))
+
+HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published
+META_BYTES = 20
+
+
+def parse_args():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--workload", default="C4", choices=["C1", "C2", "C3", "C4", "C5"])
+    ap.add_argument("--seed", type=int, default=2025)
+    ap.add_argument("--mode", default="graph", choices=["graph", "eager"],
+                    help="replay a captured HIP graph of the step (default) or launch eagerly")
+    ap.add_argument("--kernel-reps", type=int, default=50, help="launches per kernel for the per-kernel timing")
+    ap.add_argument("--cpu-seconds", type=float, default=12.0, help="target CPU time of the cpu_baseline sample")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
+    return ap.parse_args()
+
+
+def alg_bytes(T, K, H, R):
+    """Algorithmic bytes of each stage for one rank: S = T*K rows sent, R rows received."""
+    S, row = T * K, 2 * H
+    return {
+        "dispatch_send": 4 * S + T * row + S * (row + META_BYTES),
+        "dispatch_recv": 2 * R * (row + META_BYTES),
+        "combine_send": 2 * R * (row + META_BYTES),
+        "combine_recv": S * (row + META_BYTES) + 4 * S + T * row,
+    }
+
+
+def main():
+    args = parse_args()
+    if args.gpus != 1:
+        print(f"bench.py measures one rank on one GPU; --gpus {args.gpus} is not supported "
+              "(the inter-GPU exchange is outside this build)", file=sys.stderr)
+        sys.exit(2)
+
+    import numpy as np
+    import torch
+
+    from amd_distributed_2025_amd import LocalWorld, WORKLOADS, generate_world, _lib
+    from amd_distributed_2025_amd.all2all import exchange_leg
+
+    _lib.load()
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        sys.exit(2)
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+
+    wl = WORKLOADS[args.workload]
+    world = generate_world(wl, args.seed)
+    cfg = world[0][0]
+    W, K, H = len(world), cfg.experts_per_token, cfg.hidden_dim
+    data = [d.to(dev) for _, d, _, _ in world]
+
+    # ---- set-up: the whole job once, so rank 0's inbound buffers hold the peers' segments
+    lw = LocalWorld(cfg, W, device=dev)
+    ys0 = [y.clone() for y in lw.run(data)]
+    torch.cuda.synchronize()
+    a, d0, g = lw.ranks[0], data[0], lw.trace[0]
+    T = d0.num_tokens
+    R = int(g["recv_counts"].sum().item())
+    own_out = int(g["send_counts"][0].item())   # rows rank 0 sends to itself
+    own_back = int(g["back_counts"][0].item())
+    y = a._buf("y", (cfg.max_num_tokens, H), cfg.out_dtype)
+
+    def k_dispatch_send():
+        return a.dispatch_send(d0.x, d0.indices)
+
+    def k_exchange_out():
+        exchange_leg(a, a, g["send_counts"], g["send_buf"], g["send_meta"],
+                     g["recv_counts"], g["recv_buf"], g["recv_meta"], own_out)
+
+    def k_dispatch_recv():
+        return a.dispatch_recv(g["recv_counts"], g["recv_buf"], g["recv_meta"], R)
+
+    def k_expert():
+        return a.expert_scale(g["expert_x"], g["expert_num_tokens"], R)
+
+    def k_combine_send():
+        return a.combine_send(g["expert_meta"], g["expert_y"], g["expert_num_tokens"], R)
+
+    def k_exchange_back():
+        exchange_leg(a, a, g["back_counts"], g["back_buf"], g["back_meta"],
+                     g["ret_counts"], g["ret_buf"], g["ret_meta"], own_back)
+
+    def k_combine_recv():
+        a.combine_recv(y, d0.weights, g["ret_counts"], g["ret_buf"], g["ret_meta"], accumulate=False)
+
+    stages = [("dispatch_send", k_dispatch_send), ("exchange_out", k_exchange_out),
+              ("dispatch_recv", k_dispatch_recv), ("expert_standin", k_expert),
+              ("combine_send", k_combine_send), ("exchange_back", k_exchange_back),
+              ("combine_recv", k_combine_recv)]
+    path = ("dispatch_send", "dispatch_recv", "combine_send", "combine_recv")
+
+    def step():
+        for _, fn in stages:
+            fn()
+
+    # ---- whole-step timing
+    graph = None
+    if args.mode == "graph":
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            step()
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            step()
+        run_step = graph.replay
+    else:
+        run_step = step
+
+    for _ in range(args.warmup):
+        run_step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        run_step()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    ms_per_step = wall * 1e3 / args.steps
+    y_after = y[:T].clone()
+    same_as_setup = bool(torch.equal(y_after, ys0[0]))
+
+    # ---- per-kernel timing: HIP events on the launch stream around back-to-back launches
+    def time_kernel(fn, reps):
+        for _ in range(3):
+            fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        samples = []
+        for _ in range(5):
+            e0.record()
+            for _ in range(reps):
+                fn()
+            e1.record()
+            e1.synchronize()
+            samples.append(e0.elapsed_time(e1) * 1e3 / reps)
+        return statistics.median(samples), min(samples)
+
+    kern = {}
+    for name, fn in stages:
+        med, best = time_kernel(fn, args.kernel_reps)
+        kern[name] = {"us": round(med, 3), "us_min": round(best, 3)}
+    ab = alg_bytes(T, K, H, R)
+    for name in path:
+        kern[name]["alg_bytes"] = ab[name]
+        kern[name]["gbps"] = round(ab[name] / kern[name]["us"] * 1e-3, 1)
+        kern[name]["frac"] = round(kern[name]["gbps"] / HBM_PEAK_GBPS, 4)
+    hot_us = sum(kern[n]["us"] for n in path)
+    total_alg = sum(ab.values())
+    dominant = max(path, key=lambda n: kern[n]["us"])
+
+    out = {
+        "metric": "us_per_dispatch_combine",
+        "value": round(ms_per_step * 1e3, 3),
+        "unit": "us",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 6),
+        "higher_is_better": False,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16" if cfg.in_dtype == torch.bfloat16 else "f16",
+        "data": "synthetic",
+        "config": {
+            "workload": f"{args.workload}: rank 0 of world_size={W}, num_experts={cfg.num_experts}, "
+                        f"experts_per_token={K}, hidden_dim={H}, num_tokens={T}, routing={wl['routing']}, "
+                        f"weights={wl['weights']}, seed={args.seed}",
+            "rows_sent": T * K, "rows_received": R, "mode": args.mode,
+            "value_includes": "exchange and expert stand-ins",
+        },
+        "hot_path_us": round(hot_us, 3),
+        "hot_path_alg_bytes": total_alg,
+        "hot_path_gbps": round(total_alg / hot_us * 1e-3, 1),
+        "hot_path_frac_of_hbm_peak": round(total_alg / hot_us * 1e-3 / HBM_PEAK_GBPS, 4),
+        "kernels": kern,
+        "roofline": {
+            "bound": "hbm", "kernel": dominant,
+            "achieved": kern[dominant]["gbps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+            "frac": kern[dominant]["frac"], "traffic": None,
+        },
+        "result_identical_to_setup_run": same_as_setup,
+    }
+
+    # ---- CPU baseline: the row-by-row torch statement of the same step on the host cores
+    if not args.no_cpu:
+        from oracle import rowwise_torch as rw
+
+        nle, max_recv = a.num_local_experts, a.max_recv
+        x_c, idx_c, w_c = d0.x.cpu(), d0.indices.cpu(), d0.weights.cpu()
+        recv_b, recv_m = g["recv_buf"][:R].cpu(), g["recv_meta"][:R].cpu()
+        ret_b, ret_m = g["ret_buf"][: T * K].cpu(), g["ret_meta"][: T * K].cpu()
+
+        def cpu_step():
+            t = [time.perf_counter()]
+            rw.send_side(x_c, idx_c, 0, W, nle); t.append(time.perf_counter())
+            n_per, ex, em = rw.place_rows(recv_b, recv_m, nle, max_recv); t.append(time.perf_counter())
+            ey = rw.simulated_expert(ex, 0, cfg.out_dtype); t.append(time.perf_counter())
+            rw.return_side(ey, em, n_per, W); t.append(time.perf_counter())
+            yc = torch.zeros(cfg.max_num_tokens, H, dtype=cfg.out_dtype)
+            rw.accumulate(yc, w_c, ret_b, ret_m); t.append(time.perf_counter())
+            return yc[:T], [b - a_ for a_, b in zip(t, t[1:])]
+
+        runs, spent = [], 0.0
+        while spent < args.cpu_seconds and len(runs) < 50:
+            yc, parts = cpu_step()
+            runs.append(parts)
+            spent += sum(parts)
+        med = [statistics.median(r[i] for r in runs) for i in range(5)]
+        cpu_path_us = (med[0] + med[1] + med[3] + med[4]) * 1e6
+        out["cpu_baseline"] = {
+            "value": round(sum(med) * 1e6, 1), "unit": "us", "cores": torch.get_num_threads(),
+            "kind": "port",
+            "sample": f"{len(runs)} full steps of rank 0's share of {args.workload} "
+                      f"({spent:.1f} s of CPU), median per phase",
+            "hot_path_us": round(cpu_path_us, 1),
+            "expert_standin_us": round(med[2] * 1e6, 1),
+            "host_cpus": os.cpu_count(),
+            "matches_gpu_bits": bool(torch.equal(yc, y_after.cpu())),
+        }
+
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()
