@@ -23,12 +23,16 @@ namespace {
 constexpr int META = MOE_A2A_META_DIM;
 constexpr int BLOCK = 256;            // 4 wave64 per workgroup
 constexpr int NWAVES = BLOCK / 64;
-constexpr int VPT = 4;                // 16-byte vectors in flight per lane (row moves)
-constexpr int VPT_COMBINE = 2;        // vector columns per lane in the combine
 constexpr int COMBINE_CAP = 64;       // addends per token handled by the fast path
+constexpr int COMBINE_WEIGHTS = 128;  // weights of one token staged in LDS
 constexpr int COMBINE_BATCH = 8;      // addend rows loaded before accumulating
 constexpr int MAX_LOCAL_EXPERTS = 4096;  // LDS prefix table of the expert-major walkers
 constexpr int NUM_XCD = 8;
+
+// 16 bytes as a native clang vector: loads and stores of it are single
+// global_load/store_dwordx4 and the value lives in registers. (HIP's uint4 is a
+// struct whose copies become memcpy calls that can pin a local in memory.)
+typedef unsigned int b128 __attribute__((ext_vector_type(4)));
 
 // ---------------------------------------------------------------- wave / block primitives
 
@@ -99,22 +103,27 @@ __device__ __forceinline__ void dest_class(int e, int nle, int E, uint32_t magic
   }
 }
 
-template <typename V>
+// NV vectors of one row chunk held in registers. Loads are unconditional
+// (lanes past the end of the row re-read its last vector), so all of them are
+// in flight at once; only the stores are predicated.
+template <typename V, int NV>
 struct Payload {
-  V v[VPT];
+  V v[NV];
   __device__ __forceinline__ void load(const V* __restrict__ row, int base, int row_vecs) {
 #pragma unroll
-    for (int j = 0; j < VPT; ++j) {
-      int idx = base + j * BLOCK + threadIdx.x;
-      if (idx < row_vecs) v[j] = row[idx];
-    }
+    for (int j = 0; j < NV; ++j) v[j] = row[min(base + j * BLOCK + (int)threadIdx.x, row_vecs - 1)];
   }
   __device__ __forceinline__ void store(V* __restrict__ row, int base, int row_vecs) const {
 #pragma unroll
-    for (int j = 0; j < VPT; ++j) {
-      int idx = base + j * BLOCK + threadIdx.x;
+    for (int j = 0; j < NV; ++j) {
+      const int idx = base + j * BLOCK + threadIdx.x;
       if (idx < row_vecs) row[idx] = v[j];
     }
+  }
+  template <typename F>
+  __device__ __forceinline__ void map(F f) {
+#pragma unroll
+    for (int j = 0; j < NV; ++j) v[j] = f(v[j]);
   }
 };
 
@@ -124,44 +133,63 @@ __device__ __forceinline__ int sum_counts(const int* __restrict__ counts, int n)
   return s;
 }
 
-// ---------------------------------------------------------------- stage 1: dispatch, send side
+// Number of keys i in [0, n) that pass `test(key_i, i)`, summed over the lanes
+// of this thread only (reduce with block_sum). `load(i)` fetches key i; loads
+// are issued SCAN_UNROLL at a time with clamped indices so that all of them are
+// in flight before the first compare, and lanes past n are masked out.
+constexpr int SCAN_UNROLL = 8;
+template <int BLK, typename Load, typename Test>
+__device__ __forceinline__ int count_keys(int n, Load load, Test test) {
+  int cnt = 0;
+  for (int i = threadIdx.x; i < n; i += SCAN_UNROLL * BLK) {
+    int key[SCAN_UNROLL];
+#pragma unroll
+    for (int u = 0; u < SCAN_UNROLL; ++u) key[u] = load(min(i + u * BLK, n - 1));
+#pragma unroll
+    for (int u = 0; u < SCAN_UNROLL; ++u)
+      cnt += (i + u * BLK < n) ? (int)test(key[u], i + u * BLK) : 0;
+  }
+  return cnt;
+}
 
-template <typename V>
-__global__ __launch_bounds__(BLOCK) void dispatch_send_kernel(
+// ---------------------------------------------------------------- stage 1: dispatch, send side
+//
+// grid = W counting workgroups (rows per destination rank) followed by one
+// workgroup per (entry, chunk). Entry i = t*K + k goes to slot
+//   #{entries of a lower destination} + #{earlier entries of the same destination}.
+
+template <typename V, int NV>
+__global__ __launch_bounds__(BLOCK, 8) void dispatch_send_kernel(
     const V* __restrict__ x, const int* __restrict__ indices, int S, int K, int nle, int E, int W,
     uint32_t magic, int rank, int row_vecs, int chunks, V* __restrict__ send_buf,
     int* __restrict__ send_meta, int* __restrict__ send_counts, int* __restrict__ send_slot) {
   __shared__ int red[NWAVES];
   const int tid = threadIdx.x;
+  auto key = [indices](int i) { return indices[i]; };
 
-  if ((int)blockIdx.x < W) {  // rows per destination rank
+  if ((int)blockIdx.x < W) {
     const int lo = blockIdx.x * nle, hi = lo + nle - 1;
-    int c = 0;
-    for (int i = tid; i < S; i += BLOCK) {
-      int e = indices[i];
-      c += (e >= lo) & (e <= hi);
-    }
+    int c = count_keys<BLOCK>(S, key, [lo, hi](int e, int) { return (e >= lo) & (e <= hi); });
     c = block_sum(c, red);
     if (tid == 0) send_counts[blockIdx.x] = c;
+    return;
   }
 
-  const long long items = (long long)S * chunks;
-  for (long long q = xcd_contiguous(blockIdx.x, gridDim.x); q < items; q += gridDim.x) {
-    const int i = (int)(q / chunks), c = (int)(q - (long long)i * chunks);
+  const int items = S * chunks, movers = gridDim.x - W;
+  for (int q = xcd_contiguous(blockIdx.x - W, movers); q < items; q += movers) {
+    const int i = chunks == 1 ? q : q / chunks, c = q - i * chunks;
     const int e = indices[i];
     const int t = i / K, k = i - t * K;
-    const int base = c * (BLOCK * VPT);
+    const int base = c * (BLOCK * NV);
 
-    Payload<V> p;
+    Payload<V, NV> p;
     p.load(x + (size_t)t * row_vecs, base, row_vecs);
 
     int lo, hi, d;
     dest_class(e, nle, E, magic, lo, hi, d);
-    int cnt = 0;
-    for (int i2 = tid; i2 < S; i2 += BLOCK) {
-      int e2 = indices[i2];
-      cnt += (e2 < lo) | ((e2 <= hi) & (e2 >= lo) & (i2 < i));
-    }
+    const int cnt = count_keys<BLOCK>(S, key, [lo, hi, i](int e2, int i2) {
+      return (e2 < lo) | ((e2 <= hi) & (e2 >= lo) & (i2 < i));
+    });
     const int slot = block_sum(cnt, red);
 
     p.store(send_buf + (size_t)slot * row_vecs, base, row_vecs);
@@ -176,9 +204,13 @@ __global__ __launch_bounds__(BLOCK) void dispatch_send_kernel(
 }
 
 // ---------------------------------------------------------------- stage 2: dispatch, receive side
+//
+// grid = nle counting workgroups (rows per local expert) followed by one
+// workgroup per (received row, chunk). Row i goes to expert le = e % nle at
+// position #{earlier rows of the same expert}.
 
-template <typename V>
-__global__ __launch_bounds__(BLOCK) void dispatch_recv_kernel(
+template <typename V, int NV>
+__global__ __launch_bounds__(BLOCK, 8) void dispatch_recv_kernel(
     const V* __restrict__ recv_buf, const int* __restrict__ recv_meta,
     const int* __restrict__ recv_counts, int W, int nle, uint32_t magic, int max_recv,
     int row_vecs, int chunks, int* __restrict__ expert_num_tokens, V* __restrict__ expert_x,
@@ -186,29 +218,29 @@ __global__ __launch_bounds__(BLOCK) void dispatch_recv_kernel(
   __shared__ int red[NWAVES];
   const int tid = threadIdx.x;
   const int R = sum_counts(recv_counts, W);
+  auto key = [recv_meta](int i) { return recv_meta[(size_t)i * META]; };
 
-  if ((int)blockIdx.x < nle) {  // rows per local expert
-    int c = 0;
-    for (int i = tid; i < R; i += BLOCK)
-      c += floormod(recv_meta[(size_t)i * META], nle, magic) == (int)blockIdx.x;
+  if ((int)blockIdx.x < nle) {
+    const int me = blockIdx.x;
+    int c = count_keys<BLOCK>(R, key, [=](int e, int) { return floormod(e, nle, magic) == me; });
     c = block_sum(c, red);
-    if (tid == 0) expert_num_tokens[blockIdx.x] = c;
+    if (tid == 0) expert_num_tokens[me] = c;
+    return;
   }
 
-  const long long items = (long long)R * chunks;
-  for (long long q = blockIdx.x; q < items; q += gridDim.x) {
-    const int i = (int)(q / chunks), c = (int)(q - (long long)i * chunks);
-    const int base = c * (BLOCK * VPT);
+  const int items = R * chunks, movers = gridDim.x - nle;
+  for (int q = blockIdx.x - nle; q < items; q += movers) {
+    const int i = chunks == 1 ? q : q / chunks, c = q - i * chunks;
+    const int base = c * (BLOCK * NV);
 
-    Payload<V> p;
+    Payload<V, NV> p;
     p.load(recv_buf + (size_t)i * row_vecs, base, row_vecs);
 
     int m = 0;
     if (c == 0 && tid < META) m = recv_meta[(size_t)i * META + tid];
     const int le = floormod(recv_meta[(size_t)i * META], nle, magic);
-    int cnt = 0;
-    for (int i2 = tid; i2 < i; i2 += BLOCK)
-      cnt += floormod(recv_meta[(size_t)i2 * META], nle, magic) == le;
+    const int cnt =
+        count_keys<BLOCK>(i, key, [=](int e2, int) { return floormod(e2, nle, magic) == le; });
     const int pos = block_sum(cnt, red);
 
     if (pos < max_recv) {
@@ -250,20 +282,46 @@ __device__ __forceinline__ int expert_prefix(const int* __restrict__ cnt, int nl
   return total;
 }
 
-// Largest le with pre[le] <= g (g < pre[nle]); skips empty experts.
-__device__ __forceinline__ int expert_of(const int* pre, int nle, int g) {
-  int lo = 0, hi = nle;  // invariant: pre[lo] <= g < pre[hi]
-  while (hi - lo > 1) {
-    int mid = (lo + hi) >> 1;
-    if (pre[mid] <= g) lo = mid; else hi = mid;
+// Largest le in [0, nle) with pre[le] <= g, for g < pre[nle] (so empty experts
+// are skipped). Fixed-trip binary lifting: `top` is the largest power of two
+// below nle (0 when nle == 1), so several searches can run interleaved.
+__device__ __forceinline__ int expert_of(const int* pre, int nle, int top, int g) {
+  int lo = 0;
+  for (int step = top; step > 0; step >>= 1) {
+    const int c = lo + step;
+    if (c < nle && pre[c] <= g) lo = c;
   }
   return lo;
 }
 
-// ---------------------------------------------------------------- stage 3: combine, send side
+__device__ __forceinline__ int top_step(int nle) {
+  int top = 0;
+  for (int s = 1; s < nle; s <<= 1) top = s;
+  return top;
+}
 
-template <typename V>
-__global__ __launch_bounds__(BLOCK) void combine_send_kernel(
+// Key (one int of the meta row) of SCAN_UNROLL rows of the expert-major stream
+// at once: the searches advance in lock step so their LDS reads overlap.
+template <int FIELD>
+struct ExpertStreamKeys {
+  const int* pre;
+  const int* __restrict__ meta;
+  int nle, top, max_recv;
+  __device__ __forceinline__ int operator()(int g) const {
+    const int le = expert_of(pre, nle, top, g);
+    const size_t row = (size_t)le * max_recv + (g - pre[le]);
+    return meta[row * META + FIELD];
+  }
+};
+
+// ---------------------------------------------------------------- stage 3: combine, send side
+//
+// grid = W counting workgroups (rows per origin rank) followed by one workgroup
+// per (valid expert row, chunk), rows numbered g in (le, j) order. Row g with
+// origin d goes to slot #{rows of a lower origin} + #{earlier rows of origin d}.
+
+template <typename V, int NV>
+__global__ __launch_bounds__(BLOCK, 8) void combine_send_kernel(
     const V* __restrict__ expert_y, const int* __restrict__ expert_meta,
     const int* __restrict__ expert_num_tokens, int nle, int max_recv, int W, int row_vecs,
     int chunks, V* __restrict__ send_buf, int* __restrict__ send_meta,
@@ -272,38 +330,31 @@ __global__ __launch_bounds__(BLOCK) void combine_send_kernel(
   __shared__ int pre[MAX_LOCAL_EXPERTS + 1];
   const int tid = threadIdx.x;
   const int R = expert_prefix(expert_num_tokens, nle, max_recv, pre, red);
+  const ExpertStreamKeys<1> key{pre, expert_meta, nle, top_step(nle), max_recv};
 
-  if ((int)blockIdx.x < W) {  // rows per origin rank
-    int c = 0, le = 0;
-    for (int g = tid; g < R; g += BLOCK) {
-      while (g >= pre[le + 1]) ++le;
-      const size_t row = (size_t)le * max_recv + (g - pre[le]);
-      c += expert_meta[row * META + 1] == (int)blockIdx.x;
-    }
+  if ((int)blockIdx.x < W) {
+    const int me = blockIdx.x;
+    int c = count_keys<BLOCK>(R, key, [me](int d, int) { return d == me; });
     c = block_sum(c, red);
-    if (tid == 0) send_counts[blockIdx.x] = c;
+    if (tid == 0) send_counts[me] = c;
+    return;
   }
 
-  const long long items = (long long)R * chunks;
-  for (long long q = blockIdx.x; q < items; q += gridDim.x) {
-    const int g = (int)(q / chunks), c = (int)(q - (long long)g * chunks);
-    const int base = c * (BLOCK * VPT);
-    const int le = expert_of(pre, nle, g);
+  const int items = R * chunks, movers = gridDim.x - W;
+  for (int q = blockIdx.x - W; q < items; q += movers) {
+    const int g = chunks == 1 ? q : q / chunks, c = q - g * chunks;
+    const int base = c * (BLOCK * NV);
+    const int le = expert_of(pre, nle, key.top, g);
     const size_t row = (size_t)le * max_recv + (g - pre[le]);
 
-    Payload<V> p;
+    Payload<V, NV> p;
     p.load(expert_y + row * row_vecs, base, row_vecs);
 
     int m = 0;
     if (c == 0 && tid < META) m = expert_meta[row * META + tid];
     const int d = expert_meta[row * META + 1];
-    int cnt = 0, le2 = 0;
-    for (int g2 = tid; g2 < R; g2 += BLOCK) {
-      while (g2 >= pre[le2 + 1]) ++le2;
-      const size_t row2 = (size_t)le2 * max_recv + (g2 - pre[le2]);
-      const int d2 = expert_meta[row2 * META + 1];
-      cnt += (d2 < d) | ((d2 == d) & (g2 < g));
-    }
+    const int cnt = count_keys<BLOCK>(
+        R, key, [d, g](int d2, int g2) { return (d2 < d) | ((d2 == d) & (g2 < g)); });
     const int slot = block_sum(cnt, red);
 
     p.store(send_buf + (size_t)slot * row_vecs, base, row_vecs);
@@ -334,7 +385,7 @@ template <> __device__ __forceinline__ uint16_t to_b16<MOE_A2A_F16>(float f) {
 }
 
 template <typename V> struct Lanes;  // 16-bit elements held by one vector
-template <> struct Lanes<uint4> { static constexpr int N = 8; };
+template <> struct Lanes<b128> { static constexpr int N = 8; };
 template <> struct Lanes<uint16_t> { static constexpr int N = 1; };
 
 template <typename V>
@@ -352,7 +403,7 @@ __device__ __forceinline__ V pack16(const uint16_t* h) {
   if constexpr (Lanes<V>::N == 1) {
     return h[0];
   } else {
-    uint4 v;
+    b128 v;
     v.x = (uint32_t)h[0] | ((uint32_t)h[1] << 16);
     v.y = (uint32_t)h[2] | ((uint32_t)h[3] << 16);
     v.z = (uint32_t)h[4] | ((uint32_t)h[5] << 16);
@@ -371,8 +422,12 @@ __device__ __forceinline__ float combine_step(float acc, uint16_t v, float w) {
   return to_f32<DT>(to_b16<DT>(a));
 }
 
-template <typename V, int DT>
-__global__ __launch_bounds__(BLOCK) void combine_recv_kernel(
+// Workgroup of BLK lanes per (token, chunk); each lane owns NV vector columns.
+// The workgroup finds the rows addressed to its token by scanning the src_token
+// column of the arriving meta rows, orders them by arrival index, then walks
+// them in that order with all rows of a batch loaded up front.
+template <typename V, int DT, int BLK, int NV>
+__global__ __launch_bounds__(BLK) void combine_recv_kernel(
     const V* __restrict__ recv_buf, const int* __restrict__ recv_meta,
     const int* __restrict__ recv_counts, int W, const float* __restrict__ weights, int T, int K,
     int row_vecs, int chunks, V* __restrict__ out, int accumulate) {
@@ -380,69 +435,81 @@ __global__ __launch_bounds__(BLOCK) void combine_recv_kernel(
   __shared__ int hit_row[COMBINE_CAP], hit_k[COMBINE_CAP];
   __shared__ int ord_row[COMBINE_CAP];
   __shared__ float ord_w[COMBINE_CAP];
+  __shared__ float wts[COMBINE_WEIGHTS];
   __shared__ int nhit;
   const int tid = threadIdx.x;
   const int R = sum_counts(recv_counts, W);
+  const int kw = min(K, COMBINE_WEIGHTS);
 
-  const long long items = (long long)T * chunks;
-  for (long long q = blockIdx.x; q < items; q += gridDim.x) {
-    const int t = (int)(q / chunks), c = (int)(q - (long long)t * chunks);
-    const int base = c * (BLOCK * VPT_COMBINE);
+  const int items = T * chunks;
+  for (int q = blockIdx.x; q < items; q += gridDim.x) {
+    const int t = chunks == 1 ? q : q / chunks, c = q - t * chunks;
+    const int base = c * (BLK * NV);
     V* __restrict__ orow = out + (size_t)t * row_vecs;
 
-    float acc[VPT_COMBINE][N];
+    // the token's weights travel to LDS while the scan's loads are in flight
+    float wreg = 0.0f;
+    if (tid < kw) wreg = weights[(size_t)t * K + tid];
+
+    float acc[NV][N];
 #pragma unroll
-    for (int j = 0; j < VPT_COMBINE; ++j) {
-      const int idx = base + j * BLOCK + tid;
+    for (int j = 0; j < NV; ++j) {
       V o{};
-      if (accumulate && idx < row_vecs) o = orow[idx];
+      if (accumulate) o = orow[min(base + j * BLK + tid, row_vecs - 1)];
 #pragma unroll
       for (int e = 0; e < N; ++e) acc[j][e] = accumulate ? to_f32<DT>(get16(o, e)) : 0.0f;
     }
 
-    // rows addressed to token t, in arrival order
     if (tid == 0) nhit = 0;
     __syncthreads();
-    for (int i = tid; i < R; i += BLOCK) {
-      if (recv_meta[(size_t)i * META + 2] == t) {
-        const int p = atomicAdd(&nhit, 1);
-        if (p < COMBINE_CAP) {
-          hit_row[p] = i;
-          hit_k[p] = recv_meta[(size_t)i * META + 3];
+    for (int i = tid; i < R; i += SCAN_UNROLL * BLK) {
+      int key[SCAN_UNROLL];
+#pragma unroll
+      for (int u = 0; u < SCAN_UNROLL; ++u)
+        key[u] = recv_meta[(size_t)min(i + u * BLK, R - 1) * META + 2];
+#pragma unroll
+      for (int u = 0; u < SCAN_UNROLL; ++u) {
+        const int row = i + u * BLK;
+        if (row < R && key[u] == t) {
+          const int p = atomicAdd(&nhit, 1);
+          if (p < COMBINE_CAP) {
+            hit_row[p] = row;
+            hit_k[p] = recv_meta[(size_t)row * META + 3];
+          }
         }
       }
     }
+    if (tid < kw) wts[tid] = wreg;
     __syncthreads();
     const int n = nhit;
 
     if (n <= COMBINE_CAP) {
-      if (tid < n) {
+      if (tid < n) {  // order the hits by arrival index
         const int me = hit_row[tid];
         int r = 0;
         for (int b = 0; b < n; ++b) r += hit_row[b] < me;
         const int k = hit_k[tid];
         const bool ok = (k >= 0) & (k < K);
         ord_row[r] = ok ? me : -1;
-        ord_w[r] = ok ? weights[(size_t)t * K + k] : 0.0f;
+        ord_w[r] = !ok ? 0.0f : k < kw ? wts[k] : weights[(size_t)t * K + k];
       }
       __syncthreads();
       for (int a0 = 0; a0 < n; a0 += COMBINE_BATCH) {
-        V v[COMBINE_BATCH][VPT_COMBINE];
+        V v[COMBINE_BATCH][NV];
 #pragma unroll
         for (int u = 0; u < COMBINE_BATCH; ++u) {
-          const int row = (a0 + u < n) ? ord_row[a0 + u] : -1;
+          // clamped, unconditional loads keep the whole batch in flight
+          const int row = max(ord_row[min(a0 + u, n - 1)], 0);
 #pragma unroll
-          for (int j = 0; j < VPT_COMBINE; ++j) {
-            const int idx = base + j * BLOCK + tid;
-            if (row >= 0 && idx < row_vecs) v[u][j] = recv_buf[(size_t)row * row_vecs + idx];
-          }
+          for (int j = 0; j < NV; ++j)
+            v[u][j] = recv_buf[(size_t)row * row_vecs + min(base + j * BLK + tid, row_vecs - 1)];
         }
 #pragma unroll
         for (int u = 0; u < COMBINE_BATCH; ++u) {
           if (a0 + u < n && ord_row[a0 + u] >= 0) {
             const float w = ord_w[a0 + u];
 #pragma unroll
-            for (int j = 0; j < VPT_COMBINE; ++j)
+            for (int j = 0; j < NV; ++j)
 #pragma unroll
               for (int e = 0; e < N; ++e)
                 acc[j][e] = combine_step<DT>(acc[j][e], get16(v[u][j], e), w);
@@ -457,8 +524,8 @@ __global__ __launch_bounds__(BLOCK) void combine_recv_kernel(
         if (k < 0 || k >= K) continue;
         const float w = weights[(size_t)t * K + k];
 #pragma unroll
-        for (int j = 0; j < VPT_COMBINE; ++j) {
-          const int idx = base + j * BLOCK + tid;
+        for (int j = 0; j < NV; ++j) {
+          const int idx = base + j * BLK + tid;
           if (idx < row_vecs) {
             const V v = recv_buf[(size_t)i * row_vecs + idx];
 #pragma unroll
@@ -469,8 +536,8 @@ __global__ __launch_bounds__(BLOCK) void combine_recv_kernel(
     }
 
 #pragma unroll
-    for (int j = 0; j < VPT_COMBINE; ++j) {
-      const int idx = base + j * BLOCK + tid;
+    for (int j = 0; j < NV; ++j) {
+      const int idx = base + j * BLK + tid;
       if (idx < row_vecs) {
         uint16_t h[N];
 #pragma unroll
@@ -478,45 +545,45 @@ __global__ __launch_bounds__(BLOCK) void combine_recv_kernel(
         orow[idx] = pack16<V>(h);
       }
     }
-    __syncthreads();  // hit/ord lists are reused by the next item
+    __syncthreads();  // the LDS lists are reused by the next item
   }
 }
 
 // ---------------------------------------------------------------- simulated expert
 
-template <typename V, int DIN, int DOUT>
+template <typename V, int NV, int DIN, int DOUT>
 __global__ __launch_bounds__(BLOCK) void expert_scale_kernel(
     const V* __restrict__ expert_x, const int* __restrict__ expert_num_tokens, int nle,
     int max_recv, float scale, int row_vecs, int chunks, V* __restrict__ expert_y) {
-  constexpr int N = Lanes<V>::N;
   __shared__ int red[NWAVES];
   __shared__ int pre[MAX_LOCAL_EXPERTS + 1];
   const int R = expert_prefix(expert_num_tokens, nle, max_recv, pre, red);
-  const long long items = (long long)R * chunks;
-  for (long long q = blockIdx.x; q < items; q += gridDim.x) {
-    const int g = (int)(q / chunks), c = (int)(q - (long long)g * chunks);
-    const int base = c * (BLOCK * VPT);
-    const int le = expert_of(pre, nle, g);
+  const int top = top_step(nle);
+  const int items = R * chunks;
+  for (int q = blockIdx.x; q < items; q += gridDim.x) {
+    const int g = chunks == 1 ? q : q / chunks, c = q - g * chunks;
+    const int base = c * (BLOCK * NV);
+    const int le = expert_of(pre, nle, top, g);
     const size_t row = (size_t)le * max_recv + (g - pre[le]);
-    Payload<V> p;
+    Payload<V, NV> p;
     p.load(expert_x + row * row_vecs, base, row_vecs);
-#pragma unroll
-    for (int j = 0; j < VPT; ++j) {
+    p.map([scale](V v) {
+      constexpr int N = Lanes<V>::N;
       uint16_t h[N];
 #pragma unroll
       for (int e = 0; e < N; ++e) {
-        const float f = to_f32<DOUT>(to_b16<DOUT>(to_f32<DIN>(get16(p.v[j], e))));
+        const float f = to_f32<DOUT>(to_b16<DOUT>(to_f32<DIN>(get16(v, e))));
         h[e] = to_b16<DOUT>(__fmul_rn(f, scale));
       }
-      p.v[j] = pack16<V>(h);
-    }
+      return pack16<V>(h);
+    });
     p.store(expert_y + row * row_vecs, base, row_vecs);
   }
 }
 
 // ---------------------------------------------------------------- exchange stand-in
 
-template <typename V>
+template <typename V, int NV>
 __global__ __launch_bounds__(BLOCK) void exchange_local_kernel(
     const V* __restrict__ send_buf, const int* __restrict__ send_meta,
     const int* __restrict__ send_counts, int dst_rank, V* __restrict__ recv_buf,
@@ -526,11 +593,11 @@ __global__ __launch_bounds__(BLOCK) void exchange_local_kernel(
   const int src_off = sum_counts(send_counts, dst_rank);
   const int dst_off = sum_counts(recv_counts, src_rank);
   const int n = min(max(send_counts[dst_rank], 0), max(recv_counts[src_rank], 0));
-  const long long items = (long long)n * chunks;
-  for (long long q = blockIdx.x; q < items; q += gridDim.x) {
-    const int i = (int)(q / chunks), c = (int)(q - (long long)i * chunks);
-    const int base = c * (BLOCK * VPT);
-    Payload<V> p;
+  const int items = n * chunks;
+  for (int q = blockIdx.x; q < items; q += gridDim.x) {
+    const int i = chunks == 1 ? q : q / chunks, c = q - i * chunks;
+    const int base = c * (BLOCK * NV);
+    Payload<V, NV> p;
     p.load(send_buf + (size_t)(src_off + i) * row_vecs, base, row_vecs);
     p.store(recv_buf + (size_t)(dst_off + i) * row_vecs, base, row_vecs);
     if (c == 0 && tid < META)
@@ -543,6 +610,8 @@ __global__ __launch_bounds__(BLOCK) void exchange_local_kernel(
 struct Geometry {
   bool vec16;     // 16-byte vectors usable for every row buffer of the call
   int row_vecs;   // vectors (or 2-byte elements) per row
+  int nv;         // vectors per lane of a row-move workgroup: 1, 2 or 4
+  int chunks;     // workgroups per row = ceil(row_vecs / (BLOCK * nv))
   int nle;
   int max_recv;
   uint32_t magic; // ceil(2^32 / nle)
@@ -561,35 +630,55 @@ bool aligned(const void* p, size_t a) { return ((uintptr_t)p % a) == 0; }
 template <typename... P>
 bool all_aligned(size_t a, P... ptrs) { return (aligned(ptrs, a) && ...); }
 
+void row_geometry(Geometry& g, int hidden_dim, bool ptrs_16B) {
+  const long long row_bytes = 2ll * hidden_dim;
+  g.vec16 = (row_bytes % 16 == 0) && ptrs_16B;
+  g.row_vecs = g.vec16 ? (int)(row_bytes / 16) : hidden_dim;
+  g.nv = g.row_vecs <= BLOCK ? 1 : g.row_vecs <= 2 * BLOCK ? 2 : 4;
+  g.chunks = (g.row_vecs + BLOCK * g.nv - 1) / (BLOCK * g.nv);
+}
+
 template <typename... P>
 Geometry geometry(const moe_a2a_shape* s, P... row_ptrs) {
   Geometry g;
-  const long long row_bytes = 2ll * s->hidden_dim;
-  g.vec16 = (row_bytes % 16 == 0) && all_aligned(16, row_ptrs...);
-  g.row_vecs = g.vec16 ? (int)(row_bytes / 16) : s->hidden_dim;
+  row_geometry(g, s->hidden_dim, all_aligned(16, row_ptrs...));
   g.nle = s->num_experts / s->world_size;
   g.max_recv = s->max_num_tokens * s->world_size;
   g.magic = g.nle == 1 ? 0u : (uint32_t)(0xffffffffu / (uint32_t)g.nle) + 1u;
   return g;
 }
 
-int chunks_of(int row_vecs, int vpt) { return (row_vecs + BLOCK * vpt - 1) / (BLOCK * vpt); }
-
-int grid_for(long long items, int floor_blocks) {
-  const long long cap = 1 << 20;  // kernels stride over anything beyond this
+// Workgroups that move rows: one per item up to a cap the kernels stride over.
+// `items` beyond INT_MAX are rejected by the callers before this is reached.
+int mover_blocks(long long items) {
+  const long long cap = 1 << 20;
   long long g = items < cap ? items : cap;
-  if (g < floor_blocks) g = floor_blocks;
-  if (g < 1) g = 1;
-  return (int)g;
+  return (int)(g < 1 ? 1 : g);
 }
 
+bool items_fit(long long rows, int chunks) { return rows * chunks <= INT_MAX / 2; }
+
 int launch_status() { return hipGetLastError() == hipSuccess ? MOE_A2A_OK : MOE_A2A_ELAUNCH; }
+
+// Picks the <vector type, vectors per lane> instantiation for a geometry.
+#define MOE_A2A_FOR_ROW_KERNEL(G, LAUNCH)                  \
+  do {                                                     \
+    if ((G).vec16) {                                       \
+      if ((G).nv == 1) { LAUNCH(b128, 1); }                \
+      else if ((G).nv == 2) { LAUNCH(b128, 2); }           \
+      else { LAUNCH(b128, 4); }                            \
+    } else {                                               \
+      if ((G).nv == 1) { LAUNCH(uint16_t, 1); }            \
+      else if ((G).nv == 2) { LAUNCH(uint16_t, 2); }       \
+      else { LAUNCH(uint16_t, 4); }                        \
+    }                                                      \
+  } while (0)
 
 }  // namespace
 
 extern "C" {
 
-const char* moe_a2a_version(void) { return "moe_a2a 0.1 gfx950"; }
+const char* moe_a2a_version(void) { return "moe_a2a 0.2 gfx950"; }
 
 const char* moe_a2a_strerror(int status) {
   switch (status) {
@@ -607,23 +696,18 @@ int moe_a2a_dispatch_send(const moe_a2a_shape* s, const void* x, const int32_t* 
   if (!shape_ok(s) || num_tokens < 0 || num_tokens > s->max_num_tokens || !send_counts)
     return MOE_A2A_EINVAL;
   const long long S = (long long)num_tokens * s->experts_per_token;
-  if (S > INT_MAX / 8) return MOE_A2A_EINVAL;
   if (S > 0 && (!x || !indices || !send_buf || !send_meta)) return MOE_A2A_EINVAL;
   if (!all_aligned(2, x, send_buf)) return MOE_A2A_EALIGN;
   const Geometry g = geometry(s, x, send_buf);
-  const int chunks = chunks_of(g.row_vecs, VPT);
-  const int grid = grid_for(S * chunks, s->world_size);
+  if (!items_fit(S, g.chunks)) return MOE_A2A_EINVAL;
+  const int grid = s->world_size + mover_blocks(S * g.chunks);
   hipStream_t st = (hipStream_t)stream;
-  if (g.vec16)
-    dispatch_send_kernel<uint4><<<grid, BLOCK, 0, st>>>(
-        (const uint4*)x, indices, (int)S, s->experts_per_token, g.nle, s->num_experts,
-        s->world_size, g.magic, s->rank, g.row_vecs, chunks, (uint4*)send_buf, send_meta,
-        send_counts, send_slot);
-  else
-    dispatch_send_kernel<uint16_t><<<grid, BLOCK, 0, st>>>(
-        (const uint16_t*)x, indices, (int)S, s->experts_per_token, g.nle, s->num_experts,
-        s->world_size, g.magic, s->rank, g.row_vecs, chunks, (uint16_t*)send_buf, send_meta,
-        send_counts, send_slot);
+#define LAUNCH(V, NV)                                                                          \
+  dispatch_send_kernel<V, NV><<<grid, BLOCK, 0, st>>>(                                         \
+      (const V*)x, indices, (int)S, s->experts_per_token, g.nle, s->num_experts, s->world_size, \
+      g.magic, s->rank, g.row_vecs, g.chunks, (V*)send_buf, send_meta, send_counts, send_slot)
+  MOE_A2A_FOR_ROW_KERNEL(g, LAUNCH);
+#undef LAUNCH
   return launch_status();
 }
 
@@ -637,17 +721,16 @@ int moe_a2a_dispatch_recv(const moe_a2a_shape* s, const void* recv_buf, const in
   if (rows_hint > 0 && (!recv_buf || !recv_meta)) return MOE_A2A_EINVAL;
   if (!all_aligned(2, recv_buf, expert_x)) return MOE_A2A_EALIGN;
   const Geometry g = geometry(s, recv_buf, expert_x);
-  const int chunks = chunks_of(g.row_vecs, VPT);
-  const int grid = grid_for((long long)rows_hint * chunks, g.nle);
+  // the stream can hold at most nle * max_recv rows that fit the expert buffers
+  if (!items_fit((long long)g.nle * g.max_recv, g.chunks)) return MOE_A2A_EINVAL;
+  const int grid = g.nle + mover_blocks((long long)rows_hint * g.chunks);
   hipStream_t st = (hipStream_t)stream;
-  if (g.vec16)
-    dispatch_recv_kernel<uint4><<<grid, BLOCK, 0, st>>>(
-        (const uint4*)recv_buf, recv_meta, recv_counts, s->world_size, g.nle, g.magic,
-        g.max_recv, g.row_vecs, chunks, expert_num_tokens, (uint4*)expert_x, expert_meta);
-  else
-    dispatch_recv_kernel<uint16_t><<<grid, BLOCK, 0, st>>>(
-        (const uint16_t*)recv_buf, recv_meta, recv_counts, s->world_size, g.nle, g.magic,
-        g.max_recv, g.row_vecs, chunks, expert_num_tokens, (uint16_t*)expert_x, expert_meta);
+#define LAUNCH(V, NV)                                                                       \
+  dispatch_recv_kernel<V, NV><<<grid, BLOCK, 0, st>>>(                                      \
+      (const V*)recv_buf, recv_meta, recv_counts, s->world_size, g.nle, g.magic, g.max_recv, \
+      g.row_vecs, g.chunks, expert_num_tokens, (V*)expert_x, expert_meta)
+  MOE_A2A_FOR_ROW_KERNEL(g, LAUNCH);
+#undef LAUNCH
   return launch_status();
 }
 
@@ -661,17 +744,15 @@ int moe_a2a_combine_send(const moe_a2a_shape* s, const void* expert_y, const int
   if (!all_aligned(2, expert_y, send_buf)) return MOE_A2A_EALIGN;
   const Geometry g = geometry(s, expert_y, send_buf);
   if (g.nle > MAX_LOCAL_EXPERTS) return MOE_A2A_EINVAL;
-  const int chunks = chunks_of(g.row_vecs, VPT);
-  const int grid = grid_for((long long)rows_hint * chunks, s->world_size);
+  if (!items_fit((long long)g.nle * g.max_recv, g.chunks)) return MOE_A2A_EINVAL;
+  const int grid = s->world_size + mover_blocks((long long)rows_hint * g.chunks);
   hipStream_t st = (hipStream_t)stream;
-  if (g.vec16)
-    combine_send_kernel<uint4><<<grid, BLOCK, 0, st>>>(
-        (const uint4*)expert_y, expert_meta, expert_num_tokens, g.nle, g.max_recv, s->world_size,
-        g.row_vecs, chunks, (uint4*)send_buf, send_meta, send_counts);
-  else
-    combine_send_kernel<uint16_t><<<grid, BLOCK, 0, st>>>(
-        (const uint16_t*)expert_y, expert_meta, expert_num_tokens, g.nle, g.max_recv,
-        s->world_size, g.row_vecs, chunks, (uint16_t*)send_buf, send_meta, send_counts);
+#define LAUNCH(V, NV)                                                                         \
+  combine_send_kernel<V, NV><<<grid, BLOCK, 0, st>>>(                                         \
+      (const V*)expert_y, expert_meta, expert_num_tokens, g.nle, g.max_recv, s->world_size,    \
+      g.row_vecs, g.chunks, (V*)send_buf, send_meta, send_counts)
+  MOE_A2A_FOR_ROW_KERNEL(g, LAUNCH);
+#undef LAUNCH
   return launch_status();
 }
 
@@ -685,22 +766,34 @@ int moe_a2a_combine_recv(const moe_a2a_shape* s, const void* recv_buf, const int
   if (!recv_buf || !recv_meta || !weights || !out_tokens) return MOE_A2A_EINVAL;
   if (!all_aligned(2, recv_buf, out_tokens)) return MOE_A2A_EALIGN;
   const Geometry g = geometry(s, recv_buf, out_tokens);
-  const int chunks = chunks_of(g.row_vecs, VPT_COMBINE);
-  const int grid = grid_for((long long)num_tokens * chunks, 1);
+  // wide rows: one 1024-lane workgroup per token scans the arrivals once; narrower rows use
+  // 256 lanes with one or two vector columns each
+  const int blk = g.row_vecs >= 768 ? 1024 : BLOCK;
+  const int nv = blk == 1024 ? 1 : g.row_vecs <= BLOCK ? 1 : 2;
+  const int chunks = (g.row_vecs + blk * nv - 1) / (blk * nv);
+  if (!items_fit(num_tokens, chunks)) return MOE_A2A_EINVAL;
+  const int grid = mover_blocks((long long)num_tokens * chunks);
   hipStream_t st = (hipStream_t)stream;
   const int K = s->experts_per_token, W = s->world_size;
-#define MOE_A2A_LAUNCH_COMBINE(V, DT)                                                          \
-  combine_recv_kernel<V, DT><<<grid, BLOCK, 0, st>>>((const V*)recv_buf, recv_meta, recv_counts, \
-                                                     W, weights, num_tokens, K, g.row_vecs,    \
-                                                     chunks, (V*)out_tokens, accumulate)
+#define LAUNCH(V, DT, BLK, NV)                                                               \
+  combine_recv_kernel<V, DT, BLK, NV><<<grid, BLK, 0, st>>>(                                 \
+      (const V*)recv_buf, recv_meta, recv_counts, W, weights, num_tokens, K, g.row_vecs,     \
+      chunks, (V*)out_tokens, accumulate)
+#define PICK_SHAPE(V, DT)                                  \
+  do {                                                     \
+    if (blk == 1024) { LAUNCH(V, DT, 1024, 1); }           \
+    else if (nv == 1) { LAUNCH(V, DT, BLOCK, 1); }         \
+    else { LAUNCH(V, DT, BLOCK, 2); }                      \
+  } while (0)
   if (g.vec16) {
-    if (dtype == MOE_A2A_BF16) MOE_A2A_LAUNCH_COMBINE(uint4, MOE_A2A_BF16);
-    else MOE_A2A_LAUNCH_COMBINE(uint4, MOE_A2A_F16);
+    if (dtype == MOE_A2A_BF16) PICK_SHAPE(b128, MOE_A2A_BF16);
+    else PICK_SHAPE(b128, MOE_A2A_F16);
   } else {
-    if (dtype == MOE_A2A_BF16) MOE_A2A_LAUNCH_COMBINE(uint16_t, MOE_A2A_BF16);
-    else MOE_A2A_LAUNCH_COMBINE(uint16_t, MOE_A2A_F16);
+    if (dtype == MOE_A2A_BF16) PICK_SHAPE(uint16_t, MOE_A2A_BF16);
+    else PICK_SHAPE(uint16_t, MOE_A2A_F16);
   }
-#undef MOE_A2A_LAUNCH_COMBINE
+#undef PICK_SHAPE
+#undef LAUNCH
   return launch_status();
 }
 
@@ -715,29 +808,28 @@ int moe_a2a_expert_scale(const moe_a2a_shape* s, const void* expert_x,
   if (!all_aligned(2, expert_x, expert_y)) return MOE_A2A_EALIGN;
   const Geometry g = geometry(s, expert_x, expert_y);
   if (g.nle > MAX_LOCAL_EXPERTS) return MOE_A2A_EINVAL;
-  const int chunks = chunks_of(g.row_vecs, VPT);
-  const int grid = grid_for((long long)rows_hint * chunks, 1);
+  if (!items_fit((long long)g.nle * g.max_recv, g.chunks)) return MOE_A2A_EINVAL;
+  const int grid = mover_blocks((long long)rows_hint * g.chunks);
   hipStream_t st = (hipStream_t)stream;
   const float scale = (float)(1 + s->rank);
-#define MOE_A2A_LAUNCH_SCALE(V, DI, DO)                                                     \
-  expert_scale_kernel<V, DI, DO><<<grid, BLOCK, 0, st>>>((const V*)expert_x, expert_num_tokens, \
-                                                         g.nle, g.max_recv, scale, g.row_vecs,  \
-                                                         chunks, (V*)expert_y)
-#define MOE_A2A_DISPATCH_SCALE(V)                                                      \
-  do {                                                                                 \
-    if (in_dtype == MOE_A2A_BF16 && out_dtype == MOE_A2A_BF16)                         \
-      MOE_A2A_LAUNCH_SCALE(V, MOE_A2A_BF16, MOE_A2A_BF16);                             \
-    else if (in_dtype == MOE_A2A_F16 && out_dtype == MOE_A2A_F16)                      \
-      MOE_A2A_LAUNCH_SCALE(V, MOE_A2A_F16, MOE_A2A_F16);                               \
-    else if (in_dtype == MOE_A2A_F16)                                                  \
-      MOE_A2A_LAUNCH_SCALE(V, MOE_A2A_F16, MOE_A2A_BF16);                              \
-    else                                                                               \
-      MOE_A2A_LAUNCH_SCALE(V, MOE_A2A_BF16, MOE_A2A_F16);                              \
+#define LAUNCH_T(V, NV, DI, DO)                                                              \
+  expert_scale_kernel<V, NV, DI, DO><<<grid, BLOCK, 0, st>>>(                                \
+      (const V*)expert_x, expert_num_tokens, g.nle, g.max_recv, scale, g.row_vecs, g.chunks, \
+      (V*)expert_y)
+#define LAUNCH(V, NV)                                                                         \
+  do {                                                                                        \
+    if (in_dtype == MOE_A2A_BF16 && out_dtype == MOE_A2A_BF16)                                \
+      LAUNCH_T(V, NV, MOE_A2A_BF16, MOE_A2A_BF16);                                            \
+    else if (in_dtype == MOE_A2A_F16 && out_dtype == MOE_A2A_F16)                             \
+      LAUNCH_T(V, NV, MOE_A2A_F16, MOE_A2A_F16);                                              \
+    else if (in_dtype == MOE_A2A_F16)                                                         \
+      LAUNCH_T(V, NV, MOE_A2A_F16, MOE_A2A_BF16);                                             \
+    else                                                                                      \
+      LAUNCH_T(V, NV, MOE_A2A_BF16, MOE_A2A_F16);                                             \
   } while (0)
-  if (g.vec16) MOE_A2A_DISPATCH_SCALE(uint4);
-  else MOE_A2A_DISPATCH_SCALE(uint16_t);
-#undef MOE_A2A_DISPATCH_SCALE
-#undef MOE_A2A_LAUNCH_SCALE
+  MOE_A2A_FOR_ROW_KERNEL(g, LAUNCH);
+#undef LAUNCH
+#undef LAUNCH_T
   return launch_status();
 }
 
@@ -751,20 +843,17 @@ int moe_a2a_exchange_local(int32_t world_size, int32_t hidden_dim, const void* s
   if (rows_hint == 0) return MOE_A2A_OK;
   if (!send_buf || !send_meta || !recv_buf || !recv_meta) return MOE_A2A_EINVAL;
   if (!all_aligned(2, send_buf, recv_buf)) return MOE_A2A_EALIGN;
-  const long long row_bytes = 2ll * hidden_dim;
-  const bool vec16 = (row_bytes % 16 == 0) && all_aligned(16, send_buf, recv_buf);
-  const int row_vecs = vec16 ? (int)(row_bytes / 16) : hidden_dim;
-  const int chunks = chunks_of(row_vecs, VPT);
-  const int grid = grid_for((long long)rows_hint * chunks, 1);
+  Geometry g{};
+  row_geometry(g, hidden_dim, all_aligned(16, send_buf, recv_buf));
+  if (!items_fit(rows_hint, g.chunks)) return MOE_A2A_EINVAL;
+  const int grid = mover_blocks((long long)rows_hint * g.chunks);
   hipStream_t st = (hipStream_t)stream;
-  if (vec16)
-    exchange_local_kernel<uint4><<<grid, BLOCK, 0, st>>>(
-        (const uint4*)send_buf, send_meta, send_counts, dst_rank, (uint4*)recv_buf, recv_meta,
-        recv_counts, src_rank, row_vecs, chunks);
-  else
-    exchange_local_kernel<uint16_t><<<grid, BLOCK, 0, st>>>(
-        (const uint16_t*)send_buf, send_meta, send_counts, dst_rank, (uint16_t*)recv_buf,
-        recv_meta, recv_counts, src_rank, row_vecs, chunks);
+#define LAUNCH(V, NV)                                                                         \
+  exchange_local_kernel<V, NV><<<grid, BLOCK, 0, st>>>(                                       \
+      (const V*)send_buf, send_meta, send_counts, dst_rank, (V*)recv_buf, recv_meta,          \
+      recv_counts, src_rank, g.row_vecs, g.chunks)
+  MOE_A2A_FOR_ROW_KERNEL(g, LAUNCH);
+#undef LAUNCH
   return launch_status();
 }
 

@@ -165,15 +165,24 @@ def main():
 
     # ---- per-kernel timing: HIP events on the launch stream around back-to-back launches
     def time_kernel(fn, reps):
-        for _ in range(3):
+        # `reps` launches captured in one HIP graph, so the host's launch cost is not in the figure
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
             fn()
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        gr = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(gr):
+            for _ in range(reps):
+                fn()
+        gr.replay()
         torch.cuda.synchronize()
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         samples = []
-        for _ in range(5):
+        for _ in range(7):
             e0.record()
-            for _ in range(reps):
-                fn()
+            gr.replay()
             e1.record()
             e1.synchronize()
             samples.append(e0.elapsed_time(e1) * 1e3 / reps)
