@@ -1,12 +1,21 @@
 // MoE dispatch/combine for one rank on MI355X (gfx950, wave64).
 //
-// Every stage is a "ranked row move": a workgroup owns one (row, chunk) item,
-// issues the 16-byte loads of its payload first, then finds the row's
-// destination slot by COUNTING the keys that precede it in the stage's stable
-// order (a few KB of keys, L2-resident, scanned by all 256 lanes and reduced
-// with a wave64 butterfly + LDS), then stores. There are no atomics on global
-// memory, no counters to clear and no cross-workgroup dependencies, so the
-// result is the same on every run and nothing has to be zeroed between calls.
+// Stages 1-3 are "ranked row moves". A workgroup owns a group of ROWS
+// consecutive rows of its stage's input stream, one wave64 per row. Each wave
+// first issues the 16-byte loads of its whole row (up to 16 vectors per lane
+// in flight), then the workgroup finds the destination slot of all its rows
+// with ONE pass over the stage's keys: a slot is the number of keys that
+// precede the row in the stage's stable order, so every lane counts, for each
+// of the group's rows, the keys it scanned that precede that row; the counts
+// are reduced with a wave64 butterfly and a small LDS exchange; then each wave
+// stores its row. The keys are a few KB and stay in L2. There are no atomics
+// on global memory, no counters to clear and no dependencies between
+// workgroups, so results do not depend on scheduling and nothing has to be
+// zeroed between calls.
+//
+// Stage 4 (combine) gives a workgroup one token: it finds the rows addressed to
+// the token, orders them by arrival, and accumulates them with the reference's
+// per-addend rounding.
 //
 // Reference behaviour reproduced here: all2all/reference.py:68-148 (dispatch),
 // :151-234 (combine), :262 (simulated expert).
@@ -21,8 +30,12 @@
 namespace {
 
 constexpr int META = MOE_A2A_META_DIM;
-constexpr int BLOCK = 256;            // 4 wave64 per workgroup
+constexpr int BLOCK = 256;            // lanes of the block-per-row kernels and counting workgroups
 constexpr int NWAVES = BLOCK / 64;
+#ifndef MOE_A2A_ROWS
+#define MOE_A2A_ROWS 4
+#endif
+constexpr int ROWS = MOE_A2A_ROWS;    // rows (= waves) per workgroup of a ranked row move
 constexpr int COMBINE_CAP = 64;       // addends per token handled by the fast path
 constexpr int COMBINE_WEIGHTS = 128;  // weights of one token staged in LDS
 constexpr int COMBINE_BATCH = 8;      // addend rows loaded before accumulating
@@ -34,7 +47,40 @@ constexpr int NUM_XCD = 8;
 // struct whose copies become memcpy calls that can pin a local in memory.)
 typedef unsigned int b128 __attribute__((ext_vector_type(4)));
 
+// Row payload is written once and read by a later kernel, never by this one:
+// streaming (nontemporal) stores keep it from write-allocating in L2.
+#ifndef MOE_A2A_NT_STORE
+#define MOE_A2A_NT_STORE 1
+#endif
+#ifndef MOE_A2A_NT_LOAD
+#define MOE_A2A_NT_LOAD 0
+#endif
+template <typename V>
+__device__ __forceinline__ void stream_store(V* p, const V& v) {
+#if MOE_A2A_NT_STORE
+  __builtin_nontemporal_store(v, p);
+#else
+  *p = v;
+#endif
+}
+template <typename V>
+__device__ __forceinline__ V stream_load(const V* p) {
+#if MOE_A2A_NT_LOAD
+  return __builtin_nontemporal_load(p);
+#else
+  return *p;
+#endif
+}
+
 // ---------------------------------------------------------------- wave / block primitives
+
+// Workgroup barrier that orders LDS traffic only. __syncthreads() also waits
+// for every global load in flight, which would drain a row's prefetched payload
+// in the middle of the slot computation; the waves here exchange data through
+// LDS alone, so waiting for the LDS counter is enough.
+__device__ __forceinline__ void lds_barrier() {
+  asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+}
 
 __device__ __forceinline__ int wave_sum(int v) {
 #pragma unroll
@@ -42,16 +88,18 @@ __device__ __forceinline__ int wave_sum(int v) {
   return v;
 }
 
-// Sum over the workgroup; every lane gets the total. `red` is NWAVES ints of
-// LDS and may be reused right after the call returns.
+// Sum over a workgroup of NW waves; every lane gets the total. `red` is NW ints
+// of LDS and may be reused right after the call returns.
+template <int NW>
 __device__ __forceinline__ int block_sum(int v, int* red) {
   v = wave_sum(v);
+  if (NW == 1) return v;
   if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
-  __syncthreads();
+  lds_barrier();
   int s = 0;
 #pragma unroll
-  for (int w = 0; w < NWAVES; ++w) s += red[w];
-  __syncthreads();
+  for (int w = 0; w < NW; ++w) s += red[w];
+  lds_barrier();
   return s;
 }
 
@@ -111,13 +159,13 @@ struct Payload {
   V v[NV];
   __device__ __forceinline__ void load(const V* __restrict__ row, int base, int row_vecs) {
 #pragma unroll
-    for (int j = 0; j < NV; ++j) v[j] = row[min(base + j * BLOCK + (int)threadIdx.x, row_vecs - 1)];
+    for (int j = 0; j < NV; ++j) v[j] = stream_load(row + min(base + j * BLOCK + (int)threadIdx.x, row_vecs - 1));
   }
   __device__ __forceinline__ void store(V* __restrict__ row, int base, int row_vecs) const {
 #pragma unroll
     for (int j = 0; j < NV; ++j) {
       const int idx = base + j * BLOCK + threadIdx.x;
-      if (idx < row_vecs) row[idx] = v[j];
+      if (idx < row_vecs) stream_store(row + idx, v[j]);
     }
   }
   template <typename F>
@@ -134,17 +182,18 @@ __device__ __forceinline__ int sum_counts(const int* __restrict__ counts, int n)
 }
 
 // Number of keys i in [0, n) that pass `test(key_i, i)`, summed over the lanes
-// of this thread only (reduce with block_sum). `load(i)` fetches key i; loads
-// are issued SCAN_UNROLL at a time with clamped indices so that all of them are
-// in flight before the first compare, and lanes past n are masked out.
+// of this thread only (reduce with block_sum). `keys.fetch(idx, key)` loads
+// SCAN_UNROLL keys at once (indices already clamped to [0, n)), so that all
+// loads are in flight before the first compare; lanes past n are masked out.
 constexpr int SCAN_UNROLL = 8;
-template <int BLK, typename Load, typename Test>
-__device__ __forceinline__ int count_keys(int n, Load load, Test test) {
+template <int BLK, typename Keys, typename Test>
+__device__ __forceinline__ int count_keys(int n, const Keys& keys, Test test) {
   int cnt = 0;
   for (int i = threadIdx.x; i < n; i += SCAN_UNROLL * BLK) {
-    int key[SCAN_UNROLL];
+    int idx[SCAN_UNROLL], key[SCAN_UNROLL];
 #pragma unroll
-    for (int u = 0; u < SCAN_UNROLL; ++u) key[u] = load(min(i + u * BLK, n - 1));
+    for (int u = 0; u < SCAN_UNROLL; ++u) idx[u] = min(i + u * BLK, n - 1);
+    keys.fetch(idx, key);
 #pragma unroll
     for (int u = 0; u < SCAN_UNROLL; ++u)
       cnt += (i + u * BLK < n) ? (int)test(key[u], i + u * BLK) : 0;
@@ -152,53 +201,161 @@ __device__ __forceinline__ int count_keys(int n, Load load, Test test) {
   return cnt;
 }
 
+// Keys stored `stride` ints apart, key i at base[i * stride].
+struct StridedKeys {
+  const int* __restrict__ base;
+  int stride;
+  __device__ __forceinline__ void fetch(const int* idx, int* key) const {
+#pragma unroll
+    for (int u = 0; u < SCAN_UNROLL; ++u) key[u] = base[(size_t)idx[u] * stride];
+  }
+};
+
+// One row chunk held by one wave: NVW vectors per lane, vector j of lane l is
+// element base + j*64 + l of the row. Loads are unconditional and clamped, so
+// all NVW of them are in flight at once; stores are predicated.
+template <typename V, int NVW>
+struct WavePayload {
+  V v[NVW];
+  __device__ __forceinline__ void load(const V* __restrict__ row, int base, int row_vecs, int lane) {
+#pragma unroll
+    for (int j = 0; j < NVW; ++j) v[j] = stream_load(row + min(base + j * 64 + lane, row_vecs - 1));
+  }
+  __device__ __forceinline__ void store(V* __restrict__ row, int base, int row_vecs, int lane) const {
+#pragma unroll
+    for (int j = 0; j < NVW; ++j) {
+      const int idx = base + j * 64 + lane;
+      if (idx < row_vecs) stream_store(row + idx, v[j]);
+    }
+  }
+};
+
+// For each of the ROWS rows r of a group: this lane's share of the number of
+// keys i in [0, n) with test(r, key_i, i). Split in two so that the first
+// batch of key loads can be issued BEFORE the row payload (loads return in
+// issue order, so the keys arrive first and the slot is ready while the payload
+// is still in flight):  RowsScan scan(n, keys);  ...issue payload...;
+// scan.finish(keys, test, cnt);
+template <typename Keys>
+struct RowsScan {
+  static constexpr int STEP = 64 * ROWS;
+  int n, i;
+  int key[SCAN_UNROLL];
+  __device__ __forceinline__ RowsScan(int n_, const Keys& keys) : n(n_), i(threadIdx.x) {
+    if (i < n) issue(keys);
+  }
+  __device__ __forceinline__ void issue(const Keys& keys) {
+    int idx[SCAN_UNROLL];
+#pragma unroll
+    for (int u = 0; u < SCAN_UNROLL; ++u) idx[u] = min(i + u * STEP, n - 1);
+    keys.fetch(idx, key);
+  }
+  template <typename Test>
+  __device__ __forceinline__ void consume(Test test, int (&cnt)[ROWS]) const {
+#pragma unroll
+    for (int u = 0; u < SCAN_UNROLL; ++u) {
+      const int i2 = i + u * STEP;
+      if (i2 < n) {
+#pragma unroll
+        for (int r = 0; r < ROWS; ++r) cnt[r] += (int)test(r, key[u], i2);
+      }
+    }
+  }
+  // The first batch is consumed in straight-line code, apart from the loop over
+  // later batches: inside a loop the compiler must assume the keys were the last
+  // loads issued and would wait for the payload as well.
+  template <typename Test>
+  __device__ __forceinline__ void finish(const Keys& keys, Test test, int (&cnt)[ROWS]) {
+#pragma unroll
+    for (int r = 0; r < ROWS; ++r) cnt[r] = 0;
+    if (i < n) consume(test, cnt);
+    for (i += SCAN_UNROLL * STEP; i < n; i += SCAN_UNROLL * STEP) {
+      issue(keys);
+      consume(test, cnt);
+    }
+  }
+};
+
+// Total of cnt[wave] over the workgroup, returned to the lanes of that wave:
+// wave w gets the count that belongs to the group's row w. `part` is
+// ROWS*ROWS ints of LDS, reusable after the call.
+__device__ __forceinline__ int rows_reduce(const int (&cnt)[ROWS], int* part, int wave, int lane) {
+  if (ROWS == 1) return wave_sum(cnt[0]);
+#pragma unroll
+  for (int r = 0; r < ROWS; ++r) {
+    const int s = wave_sum(cnt[r]);
+    if (lane == 0) part[wave * ROWS + r] = s;
+  }
+  lds_barrier();
+  int mine = 0;
+#pragma unroll
+  for (int w = 0; w < ROWS; ++w) mine += part[w * ROWS + wave];
+  lds_barrier();
+  return mine;
+}
+
 // ---------------------------------------------------------------- stage 1: dispatch, send side
 //
 // grid = W counting workgroups (rows per destination rank) followed by one
-// workgroup per (entry, chunk). Entry i = t*K + k goes to slot
+// workgroup per (group of ROWS entries, chunk). Entry i = t*K + k goes to slot
 //   #{entries of a lower destination} + #{earlier entries of the same destination}.
 
-template <typename V, int NV>
-__global__ __launch_bounds__(BLOCK, 8) void dispatch_send_kernel(
+template <typename V, int NVW>
+__global__ __launch_bounds__(64 * ROWS) void dispatch_send_kernel(
     const V* __restrict__ x, const int* __restrict__ indices, int S, int K, int nle, int E, int W,
     uint32_t magic, int rank, int row_vecs, int chunks, V* __restrict__ send_buf,
     int* __restrict__ send_meta, int* __restrict__ send_counts, int* __restrict__ send_slot) {
-  __shared__ int red[NWAVES];
-  const int tid = threadIdx.x;
-  auto key = [indices](int i) { return indices[i]; };
+  __shared__ int part[ROWS * ROWS];
+  __shared__ int s_lo[ROWS], s_hi[ROWS];
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const StridedKeys key{indices, 1};
 
   if ((int)blockIdx.x < W) {
     const int lo = blockIdx.x * nle, hi = lo + nle - 1;
-    int c = count_keys<BLOCK>(S, key, [lo, hi](int e, int) { return (e >= lo) & (e <= hi); });
-    c = block_sum(c, red);
+    int c = count_keys<64 * ROWS>(S, key, [lo, hi](int e, int) { return (e >= lo) & (e <= hi); });
+    c = block_sum<ROWS>(c, part);
     if (tid == 0) send_counts[blockIdx.x] = c;
     return;
   }
 
-  const int items = S * chunks, movers = gridDim.x - W;
+  const int groups = (S + ROWS - 1) / ROWS;
+  const int items = groups * chunks, movers = gridDim.x - W;
   for (int q = xcd_contiguous(blockIdx.x - W, movers); q < items; q += movers) {
-    const int i = chunks == 1 ? q : q / chunks, c = q - i * chunks;
-    const int e = indices[i];
-    const int t = i / K, k = i - t * K;
-    const int base = c * (BLOCK * NV);
+    const int grp = chunks == 1 ? q : q / chunks, c = q - grp * chunks;
+    const int i = grp * ROWS + wave;
+    const bool valid = i < S;
+    const int ic = min(i, S - 1);
+    const int e = indices[ic];
+    const int t = ic / K, k = ic - t * K;
+    const int base = c * (64 * NVW);
 
-    Payload<V, NV> p;
-    p.load(x + (size_t)t * row_vecs, base, row_vecs);
+    RowsScan<StridedKeys> scan(S, key);
+    WavePayload<V, NVW> p;
+    p.load(x + (size_t)t * row_vecs, base, row_vecs, lane);
 
     int lo, hi, d;
     dest_class(e, nle, E, magic, lo, hi, d);
-    const int cnt = count_keys<BLOCK>(S, key, [lo, hi, i](int e2, int i2) {
-      return (e2 < lo) | ((e2 <= hi) & (e2 >= lo) & (i2 < i));
-    });
-    const int slot = block_sum(cnt, red);
+    if (lane == 0) { s_lo[wave] = lo; s_hi[wave] = hi; }
+    lds_barrier();
+    int rlo[ROWS], rhi[ROWS];
+#pragma unroll
+    for (int r = 0; r < ROWS; ++r) { rlo[r] = s_lo[r]; rhi[r] = s_hi[r]; }
+    const int i0 = grp * ROWS;
+    int cnt[ROWS];
+    scan.finish(key, [&](int r, int e2, int i2) {
+      return (e2 < rlo[r]) | ((e2 <= rhi[r]) & (e2 >= rlo[r]) & (i2 < i0 + r));
+    }, cnt);
+    const int slot = rows_reduce(cnt, part, wave, lane);
 
-    p.store(send_buf + (size_t)slot * row_vecs, base, row_vecs);
-    if (c == 0) {
-      if (tid < META) {
-        int m = tid == 0 ? e : tid == 1 ? rank : tid == 2 ? t : tid == 3 ? k : 0;
-        send_meta[(size_t)slot * META + tid] = m;
+    if (valid) {
+      p.store(send_buf + (size_t)slot * row_vecs, base, row_vecs, lane);
+      if (c == 0) {
+        if (lane < META) {
+          int m = lane == 0 ? e : lane == 1 ? rank : lane == 2 ? t : lane == 3 ? k : 0;
+          send_meta[(size_t)slot * META + lane] = m;
+        }
+        if (lane == 0 && send_slot) send_slot[i] = slot;
       }
-      if (tid == 0 && send_slot) send_slot[i] = slot;
     }
   }
 }
@@ -206,47 +363,63 @@ __global__ __launch_bounds__(BLOCK, 8) void dispatch_send_kernel(
 // ---------------------------------------------------------------- stage 2: dispatch, receive side
 //
 // grid = nle counting workgroups (rows per local expert) followed by one
-// workgroup per (received row, chunk). Row i goes to expert le = e % nle at
-// position #{earlier rows of the same expert}.
+// workgroup per (group of ROWS received rows, chunk). Row i goes to expert
+// le = e % nle at position #{earlier rows of the same expert}.
 
-template <typename V, int NV>
-__global__ __launch_bounds__(BLOCK, 8) void dispatch_recv_kernel(
+template <typename V, int NVW>
+__global__ __launch_bounds__(64 * ROWS) void dispatch_recv_kernel(
     const V* __restrict__ recv_buf, const int* __restrict__ recv_meta,
     const int* __restrict__ recv_counts, int W, int nle, uint32_t magic, int max_recv,
     int row_vecs, int chunks, int* __restrict__ expert_num_tokens, V* __restrict__ expert_x,
     int* __restrict__ expert_meta) {
-  __shared__ int red[NWAVES];
-  const int tid = threadIdx.x;
+  __shared__ int part[ROWS * ROWS];
+  __shared__ int s_le[ROWS];
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const int R = sum_counts(recv_counts, W);
-  auto key = [recv_meta](int i) { return recv_meta[(size_t)i * META]; };
+  const StridedKeys key{recv_meta, META};
 
   if ((int)blockIdx.x < nle) {
     const int me = blockIdx.x;
-    int c = count_keys<BLOCK>(R, key, [=](int e, int) { return floormod(e, nle, magic) == me; });
-    c = block_sum(c, red);
+    int c = count_keys<64 * ROWS>(R, key, [=](int e, int) { return floormod(e, nle, magic) == me; });
+    c = block_sum<ROWS>(c, part);
     if (tid == 0) expert_num_tokens[me] = c;
     return;
   }
 
-  const int items = R * chunks, movers = gridDim.x - nle;
+  const int groups = (R + ROWS - 1) / ROWS;
+  const int items = groups * chunks, movers = gridDim.x - nle;
   for (int q = blockIdx.x - nle; q < items; q += movers) {
-    const int i = chunks == 1 ? q : q / chunks, c = q - i * chunks;
-    const int base = c * (BLOCK * NV);
+    const int grp = chunks == 1 ? q : q / chunks, c = q - grp * chunks;
+    const int i = grp * ROWS + wave;
+    const bool valid = i < R;
+    const int ic = min(i, R - 1);
+    const int base = c * (64 * NVW);
 
-    Payload<V, NV> p;
-    p.load(recv_buf + (size_t)i * row_vecs, base, row_vecs);
-
+    const int i0 = grp * ROWS;
     int m = 0;
-    if (c == 0 && tid < META) m = recv_meta[(size_t)i * META + tid];
-    const int le = floormod(recv_meta[(size_t)i * META], nle, magic);
-    const int cnt =
-        count_keys<BLOCK>(i, key, [=](int e2, int) { return floormod(e2, nle, magic) == le; });
-    const int pos = block_sum(cnt, red);
+    if (c == 0 && lane < META) m = recv_meta[(size_t)ic * META + lane];
+    const int e = recv_meta[(size_t)ic * META];
+    // only rows before the group's last row can precede any of its rows
+    RowsScan<StridedKeys> scan(min(i0 + ROWS - 1, R), key);
+    WavePayload<V, NVW> p;
+    p.load(recv_buf + (size_t)ic * row_vecs, base, row_vecs, lane);
 
-    if (pos < max_recv) {
+    const int le = floormod(e, nle, magic);
+    if (lane == 0) s_le[wave] = le;
+    lds_barrier();
+    int rle[ROWS];
+#pragma unroll
+    for (int r = 0; r < ROWS; ++r) rle[r] = s_le[r];
+    int cnt[ROWS];
+    scan.finish(key, [&](int r, int e2, int i2) {
+      return (floormod(e2, nle, magic) == rle[r]) & (i2 < i0 + r);
+    }, cnt);
+    const int pos = rows_reduce(cnt, part, wave, lane);
+
+    if (valid && pos < max_recv) {
       const size_t row = (size_t)le * max_recv + pos;
-      p.store(expert_x + row * row_vecs, base, row_vecs);
-      if (c == 0 && tid < META) expert_meta[row * META + tid] = m;
+      p.store(expert_x + row * row_vecs, base, row_vecs, lane);
+      if (c == 0 && lane < META) expert_meta[row * META + lane] = m;
     }
   }
 }
@@ -256,19 +429,20 @@ __global__ __launch_bounds__(BLOCK, 8) void dispatch_recv_kernel(
 // pre[0..nle] = exclusive prefix of min(cnt[le], max_recv); returns the total.
 // Each lane owns a contiguous run of experts; runs are combined by a wave64
 // scan and a scan over the wave totals.
+template <int NW>
 __device__ __forceinline__ int expert_prefix(const int* __restrict__ cnt, int nle, int max_recv,
                                              int* pre, int* red) {
   const int tid = threadIdx.x;
-  const int per = (nle + BLOCK - 1) / BLOCK;
+  const int per = (nle + 64 * NW - 1) / (64 * NW);
   const int b = min(tid * per, nle), e = min(b + per, nle);
   int s = 0;
   for (int i = b; i < e; ++i) s += min(max(cnt[i], 0), max_recv);
   const int inc = wave_inclusive_scan(s);
   if ((tid & 63) == 63) red[tid >> 6] = inc;
-  __syncthreads();
+  lds_barrier();
   int off = 0, total = 0;
 #pragma unroll
-  for (int w = 0; w < NWAVES; ++w) {
+  for (int w = 0; w < NW; ++w) {
     if (w < (tid >> 6)) off += red[w];
     total += red[w];
   }
@@ -278,7 +452,7 @@ __device__ __forceinline__ int expert_prefix(const int* __restrict__ cnt, int nl
     run += min(max(cnt[i], 0), max_recv);
   }
   if (tid == 0) pre[nle] = total;
-  __syncthreads();
+  lds_barrier();
   return total;
 }
 
@@ -300,127 +474,176 @@ __device__ __forceinline__ int top_step(int nle) {
   return top;
 }
 
-// Key (one int of the meta row) of SCAN_UNROLL rows of the expert-major stream
-// at once: the searches advance in lock step so their LDS reads overlap.
+// Keys (int FIELD of the meta row) of rows of the expert-major stream, row g
+// being the g-th valid row in (le, j) order. The SCAN_UNROLL searches of one
+// fetch advance in lock step, so their LDS reads overlap instead of chaining.
 template <int FIELD>
 struct ExpertStreamKeys {
-  const int* pre;
+  const int* pre;  // LDS, nle + 1 entries, pre[nle] = number of rows
   const int* __restrict__ meta;
   int nle, top, max_recv;
-  __device__ __forceinline__ int operator()(int g) const {
-    const int le = expert_of(pre, nle, top, g);
-    const size_t row = (size_t)le * max_recv + (g - pre[le]);
-    return meta[row * META + FIELD];
+  __device__ __forceinline__ void fetch(const int* g, int* key) const {
+    int le[SCAN_UNROLL];
+#pragma unroll
+    for (int u = 0; u < SCAN_UNROLL; ++u) le[u] = 0;
+    for (int step = top; step > 0; step >>= 1) {
+#pragma unroll
+      for (int u = 0; u < SCAN_UNROLL; ++u) {
+        const int c = min(le[u] + step, nle);  // pre[nle] > g: never taken
+        le[u] = pre[c] <= g[u] ? c : le[u];
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < SCAN_UNROLL; ++u) {
+      const size_t row = (size_t)le[u] * max_recv + (g[u] - pre[le[u]]);
+      key[u] = meta[row * META + FIELD];
+    }
   }
 };
 
 // ---------------------------------------------------------------- stage 3: combine, send side
 //
 // grid = W counting workgroups (rows per origin rank) followed by one workgroup
-// per (valid expert row, chunk), rows numbered g in (le, j) order. Row g with
-// origin d goes to slot #{rows of a lower origin} + #{earlier rows of origin d}.
+// per (group of ROWS valid expert rows, chunk), rows numbered g in (le, j)
+// order. Row g with origin d goes to slot
+//   #{rows of a lower origin} + #{earlier rows of origin d}.
 
-template <typename V, int NV>
-__global__ __launch_bounds__(BLOCK, 8) void combine_send_kernel(
+template <typename V, int NVW>
+__global__ __launch_bounds__(64 * ROWS) void combine_send_kernel(
     const V* __restrict__ expert_y, const int* __restrict__ expert_meta,
     const int* __restrict__ expert_num_tokens, int nle, int max_recv, int W, int row_vecs,
     int chunks, V* __restrict__ send_buf, int* __restrict__ send_meta,
     int* __restrict__ send_counts) {
-  __shared__ int red[NWAVES];
+  __shared__ int part[ROWS * ROWS];
+  __shared__ int s_d[ROWS];
   __shared__ int pre[MAX_LOCAL_EXPERTS + 1];
-  const int tid = threadIdx.x;
-  const int R = expert_prefix(expert_num_tokens, nle, max_recv, pre, red);
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int R = expert_prefix<ROWS>(expert_num_tokens, nle, max_recv, pre, part);
   const ExpertStreamKeys<1> key{pre, expert_meta, nle, top_step(nle), max_recv};
 
   if ((int)blockIdx.x < W) {
     const int me = blockIdx.x;
-    int c = count_keys<BLOCK>(R, key, [me](int d, int) { return d == me; });
-    c = block_sum(c, red);
+    int c = count_keys<64 * ROWS>(R, key, [me](int d, int) { return d == me; });
+    c = block_sum<ROWS>(c, part);
     if (tid == 0) send_counts[me] = c;
     return;
   }
 
-  const int items = R * chunks, movers = gridDim.x - W;
+  const int groups = (R + ROWS - 1) / ROWS;
+  const int items = groups * chunks, movers = gridDim.x - W;
   for (int q = blockIdx.x - W; q < items; q += movers) {
-    const int g = chunks == 1 ? q : q / chunks, c = q - g * chunks;
-    const int base = c * (BLOCK * NV);
-    const int le = expert_of(pre, nle, key.top, g);
-    const size_t row = (size_t)le * max_recv + (g - pre[le]);
-
-    Payload<V, NV> p;
-    p.load(expert_y + row * row_vecs, base, row_vecs);
+    const int grp = chunks == 1 ? q : q / chunks, c = q - grp * chunks;
+    const int g = grp * ROWS + wave;
+    const bool valid = g < R;
+    const int gc = min(g, R - 1);
+    const int base = c * (64 * NVW);
+    const int le = expert_of(pre, nle, key.top, gc);
+    const size_t row = (size_t)le * max_recv + (gc - pre[le]);
 
     int m = 0;
-    if (c == 0 && tid < META) m = expert_meta[row * META + tid];
+    if (c == 0 && lane < META) m = expert_meta[row * META + lane];
     const int d = expert_meta[row * META + 1];
-    const int cnt = count_keys<BLOCK>(
-        R, key, [d, g](int d2, int g2) { return (d2 < d) | ((d2 == d) & (g2 < g)); });
-    const int slot = block_sum(cnt, red);
+    RowsScan<ExpertStreamKeys<1>> scan(R, key);
+    WavePayload<V, NVW> p;
+    p.load(expert_y + row * row_vecs, base, row_vecs, lane);
 
-    p.store(send_buf + (size_t)slot * row_vecs, base, row_vecs);
-    if (c == 0 && tid < META) send_meta[(size_t)slot * META + tid] = m;
+    if (lane == 0) s_d[wave] = d;
+    lds_barrier();
+    int rd[ROWS];
+#pragma unroll
+    for (int r = 0; r < ROWS; ++r) rd[r] = s_d[r];
+    const int g0 = grp * ROWS;
+    int cnt[ROWS];
+    scan.finish(key, [&](int r, int d2, int g2) {
+      return (d2 < rd[r]) | ((d2 == rd[r]) & (g2 < g0 + r));
+    }, cnt);
+    const int slot = rows_reduce(cnt, part, wave, lane);
+
+    if (valid) {
+      p.store(send_buf + (size_t)slot * row_vecs, base, row_vecs, lane);
+      if (c == 0 && lane < META) send_meta[(size_t)slot * META + lane] = m;
+    }
   }
 }
 
 // ---------------------------------------------------------------- 16-bit float helpers
+//
+// Element arithmetic works on 32-bit words holding two 16-bit elements (low
+// half = even element), so that the gfx950 pair conversion v_cvt_pk_bf16_f32
+// (round to nearest even) does the rounding of both in one instruction.
+// A NaN keeps whatever payload the hardware gives it while it is being
+// accumulated; bf16 results are canonicalised to 0x7fc0 (what torch stores for
+// any NaN) where they are written out.
 
-template <int DT> __device__ __forceinline__ float to_f32(uint16_t b);
-template <> __device__ __forceinline__ float to_f32<MOE_A2A_BF16>(uint16_t b) {
-  return __uint_as_float((uint32_t)b << 16);
-}
-template <> __device__ __forceinline__ float to_f32<MOE_A2A_F16>(uint16_t b) {
-  return __half2float(__ushort_as_half(b));
-}
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
 
-// Round to nearest even, the conversion torch applies when it stores a float
-// into a 16-bit tensor.
-template <int DT> __device__ __forceinline__ uint16_t to_b16(float f);
-template <> __device__ __forceinline__ uint16_t to_b16<MOE_A2A_BF16>(float f) {
-  uint32_t u = __float_as_uint(f);
-  if ((u & 0x7fffffffu) > 0x7f800000u) return 0x7fc0;
-  return (uint16_t)((u + 0x7fffu + ((u >> 16) & 1u)) >> 16);
-}
-template <> __device__ __forceinline__ uint16_t to_b16<MOE_A2A_F16>(float f) {
-  return __half_as_ushort(__float2half_rn(f));
-}
-
-template <typename V> struct Lanes;  // 16-bit elements held by one vector
-template <> struct Lanes<b128> { static constexpr int N = 8; };
-template <> struct Lanes<uint16_t> { static constexpr int N = 1; };
-
-template <typename V>
-__device__ __forceinline__ uint16_t get16(const V& v, int e) {
-  if constexpr (Lanes<V>::N == 1) {
-    return v;
-  } else {
-    const uint32_t w = e < 2 ? v.x : e < 4 ? v.y : e < 6 ? v.z : v.w;
-    return (uint16_t)((e & 1) ? (w >> 16) : (w & 0xffffu));
+template <int DT> struct Pair16;
+template <> struct Pair16<MOE_A2A_BF16> {
+  static __device__ __forceinline__ float lo(uint32_t w) { return __uint_as_float(w << 16); }
+  static __device__ __forceinline__ float hi(uint32_t w) { return __uint_as_float(w & 0xffff0000u); }
+  static __device__ __forceinline__ uint32_t round(float a, float b) {
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(f32x2{a, b}, bf16x2));
   }
+  static __device__ __forceinline__ uint32_t canonical(uint32_t w) {
+    if ((w & 0x7fffu) > 0x7f80u) w = (w & 0xffff0000u) | 0x7fc0u;
+    if ((w & 0x7fff0000u) > 0x7f800000u) w = (w & 0x0000ffffu) | 0x7fc00000u;
+    return w;
+  }
+};
+template <> struct Pair16<MOE_A2A_F16> {
+  static __device__ __forceinline__ float lo(uint32_t w) {
+    return (float)__builtin_bit_cast(f16x2, w).x;
+  }
+  static __device__ __forceinline__ float hi(uint32_t w) {
+    return (float)__builtin_bit_cast(f16x2, w).y;
+  }
+  static __device__ __forceinline__ uint32_t round(float a, float b) {
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(f32x2{a, b}, f16x2));
+  }
+  static __device__ __forceinline__ uint32_t canonical(uint32_t w) { return w; }
+};
+
+template <typename V> struct Words;  // 32-bit words (element pairs) per vector
+template <> struct Words<b128> { static constexpr int N = 4; };
+template <> struct Words<uint16_t> { static constexpr int N = 1; };  // one element, high half unused
+
+template <typename V>
+__device__ __forceinline__ uint32_t get_word(const V& v, int i) {
+  if constexpr (Words<V>::N == 1) return v;
+  else return v[i];
 }
 
 template <typename V>
-__device__ __forceinline__ V pack16(const uint16_t* h) {
-  if constexpr (Lanes<V>::N == 1) {
-    return h[0];
+__device__ __forceinline__ V from_words(const uint32_t* w) {
+  if constexpr (Words<V>::N == 1) {
+    return (uint16_t)w[0];
   } else {
     b128 v;
-    v.x = (uint32_t)h[0] | ((uint32_t)h[1] << 16);
-    v.y = (uint32_t)h[2] | ((uint32_t)h[3] << 16);
-    v.z = (uint32_t)h[4] | ((uint32_t)h[5] << 16);
-    v.w = (uint32_t)h[6] | ((uint32_t)h[7] << 16);
+    v.x = w[0]; v.y = w[1]; v.z = w[2]; v.w = w[3];
     return v;
   }
 }
 
 // ---------------------------------------------------------------- stage 4: combine, receive side
 
-// One step of `out[t] += row.float() * w` on a 16-bit accumulator.
+// A running row sum: two floats per word, each always exactly representable in
+// the 16-bit type. step() is one `out[t] += row.float() * w` of the reference:
+//   p = RN32(f32(v) * w);  a = RN32(acc + p);  acc = RN16(a)
 template <int DT>
-__device__ __forceinline__ float combine_step(float acc, uint16_t v, float w) {
-  const float p = __fmul_rn(to_f32<DT>(v), w);
-  const float a = __fadd_rn(acc, p);
-  return to_f32<DT>(to_b16<DT>(a));
-}
+struct PairAcc {
+  float lo, hi;
+  __device__ __forceinline__ void set(uint32_t w) { lo = Pair16<DT>::lo(w); hi = Pair16<DT>::hi(w); }
+  __device__ __forceinline__ void step(uint32_t v, float w) {
+    const float a = __fadd_rn(lo, __fmul_rn(Pair16<DT>::lo(v), w));
+    const float b = __fadd_rn(hi, __fmul_rn(Pair16<DT>::hi(v), w));
+    set(Pair16<DT>::round(a, b));
+  }
+  __device__ __forceinline__ uint32_t word() const {
+    return Pair16<DT>::canonical(Pair16<DT>::round(lo, hi));
+  }
+};
 
 // Workgroup of BLK lanes per (token, chunk); each lane owns NV vector columns.
 // The workgroup finds the rows addressed to its token by scanning the src_token
@@ -431,7 +654,7 @@ __global__ __launch_bounds__(BLK) void combine_recv_kernel(
     const V* __restrict__ recv_buf, const int* __restrict__ recv_meta,
     const int* __restrict__ recv_counts, int W, const float* __restrict__ weights, int T, int K,
     int row_vecs, int chunks, V* __restrict__ out, int accumulate) {
-  constexpr int N = Lanes<V>::N;
+  constexpr int N = Words<V>::N;
   __shared__ int hit_row[COMBINE_CAP], hit_k[COMBINE_CAP];
   __shared__ int ord_row[COMBINE_CAP];
   __shared__ float ord_w[COMBINE_CAP];
@@ -451,22 +674,25 @@ __global__ __launch_bounds__(BLK) void combine_recv_kernel(
     float wreg = 0.0f;
     if (tid < kw) wreg = weights[(size_t)t * K + tid];
 
-    float acc[NV][N];
+    PairAcc<DT> acc[NV][N];
 #pragma unroll
     for (int j = 0; j < NV; ++j) {
       V o{};
       if (accumulate) o = orow[min(base + j * BLK + tid, row_vecs - 1)];
 #pragma unroll
-      for (int e = 0; e < N; ++e) acc[j][e] = accumulate ? to_f32<DT>(get16(o, e)) : 0.0f;
+      for (int e = 0; e < N; ++e) acc[j][e].set(get_word(o, e));
     }
 
     if (tid == 0) nhit = 0;
-    __syncthreads();
+    lds_barrier();
     for (int i = tid; i < R; i += SCAN_UNROLL * BLK) {
-      int key[SCAN_UNROLL];
+      int key[SCAN_UNROLL], kk[SCAN_UNROLL];
 #pragma unroll
-      for (int u = 0; u < SCAN_UNROLL; ++u)
-        key[u] = recv_meta[(size_t)min(i + u * BLK, R - 1) * META + 2];
+      for (int u = 0; u < SCAN_UNROLL; ++u) {
+        const int* m = recv_meta + (size_t)min(i + u * BLK, R - 1) * META;
+        key[u] = m[2];
+        kk[u] = m[3];
+      }
 #pragma unroll
       for (int u = 0; u < SCAN_UNROLL; ++u) {
         const int row = i + u * BLK;
@@ -474,13 +700,13 @@ __global__ __launch_bounds__(BLK) void combine_recv_kernel(
           const int p = atomicAdd(&nhit, 1);
           if (p < COMBINE_CAP) {
             hit_row[p] = row;
-            hit_k[p] = recv_meta[(size_t)row * META + 3];
+            hit_k[p] = kk[u];
           }
         }
       }
     }
     if (tid < kw) wts[tid] = wreg;
-    __syncthreads();
+    lds_barrier();
     const int n = nhit;
 
     if (n <= COMBINE_CAP) {
@@ -493,7 +719,7 @@ __global__ __launch_bounds__(BLK) void combine_recv_kernel(
         ord_row[r] = ok ? me : -1;
         ord_w[r] = !ok ? 0.0f : k < kw ? wts[k] : weights[(size_t)t * K + k];
       }
-      __syncthreads();
+      lds_barrier();
       for (int a0 = 0; a0 < n; a0 += COMBINE_BATCH) {
         V v[COMBINE_BATCH][NV];
 #pragma unroll
@@ -511,8 +737,7 @@ __global__ __launch_bounds__(BLK) void combine_recv_kernel(
 #pragma unroll
             for (int j = 0; j < NV; ++j)
 #pragma unroll
-              for (int e = 0; e < N; ++e)
-                acc[j][e] = combine_step<DT>(acc[j][e], get16(v[u][j], e), w);
+              for (int e = 0; e < N; ++e) acc[j][e].step(get_word(v[u][j], e), w);
           }
         }
       }
@@ -529,7 +754,7 @@ __global__ __launch_bounds__(BLK) void combine_recv_kernel(
           if (idx < row_vecs) {
             const V v = recv_buf[(size_t)i * row_vecs + idx];
 #pragma unroll
-            for (int e = 0; e < N; ++e) acc[j][e] = combine_step<DT>(acc[j][e], get16(v, e), w);
+            for (int e = 0; e < N; ++e) acc[j][e].step(get_word(v, e), w);
           }
         }
       }
@@ -539,13 +764,13 @@ __global__ __launch_bounds__(BLK) void combine_recv_kernel(
     for (int j = 0; j < NV; ++j) {
       const int idx = base + j * BLK + tid;
       if (idx < row_vecs) {
-        uint16_t h[N];
+        uint32_t h[N];
 #pragma unroll
-        for (int e = 0; e < N; ++e) h[e] = to_b16<DT>(acc[j][e]);
-        orow[idx] = pack16<V>(h);
+        for (int e = 0; e < N; ++e) h[e] = acc[j][e].word();
+        orow[idx] = from_words<V>(h);
       }
     }
-    __syncthreads();  // the LDS lists are reused by the next item
+    lds_barrier();  // the LDS lists are reused by the next item
   }
 }
 
@@ -557,7 +782,7 @@ __global__ __launch_bounds__(BLOCK) void expert_scale_kernel(
     int max_recv, float scale, int row_vecs, int chunks, V* __restrict__ expert_y) {
   __shared__ int red[NWAVES];
   __shared__ int pre[MAX_LOCAL_EXPERTS + 1];
-  const int R = expert_prefix(expert_num_tokens, nle, max_recv, pre, red);
+  const int R = expert_prefix<NWAVES>(expert_num_tokens, nle, max_recv, pre, red);
   const int top = top_step(nle);
   const int items = R * chunks;
   for (int q = blockIdx.x; q < items; q += gridDim.x) {
@@ -568,14 +793,17 @@ __global__ __launch_bounds__(BLOCK) void expert_scale_kernel(
     Payload<V, NV> p;
     p.load(expert_x + row * row_vecs, base, row_vecs);
     p.map([scale](V v) {
-      constexpr int N = Lanes<V>::N;
-      uint16_t h[N];
+      constexpr int N = Words<V>::N;
+      uint32_t h[N];
 #pragma unroll
       for (int e = 0; e < N; ++e) {
-        const float f = to_f32<DOUT>(to_b16<DOUT>(to_f32<DIN>(get16(v, e))));
-        h[e] = to_b16<DOUT>(__fmul_rn(f, scale));
+        const uint32_t w = get_word(v, e);
+        // .to(out_dtype), then times (1 + rank) in float32, rounded once
+        const uint32_t o = Pair16<DOUT>::round(Pair16<DIN>::lo(w), Pair16<DIN>::hi(w));
+        h[e] = Pair16<DOUT>::canonical(Pair16<DOUT>::round(__fmul_rn(Pair16<DOUT>::lo(o), scale),
+                                                           __fmul_rn(Pair16<DOUT>::hi(o), scale)));
       }
-      return pack16<V>(h);
+      return from_words<V>(h);
     });
     p.store(expert_y + row * row_vecs, base, row_vecs);
   }
@@ -610,8 +838,10 @@ __global__ __launch_bounds__(BLOCK) void exchange_local_kernel(
 struct Geometry {
   bool vec16;     // 16-byte vectors usable for every row buffer of the call
   int row_vecs;   // vectors (or 2-byte elements) per row
-  int nv;         // vectors per lane of a row-move workgroup: 1, 2 or 4
-  int chunks;     // workgroups per row = ceil(row_vecs / (BLOCK * nv))
+  int nv;         // block-per-row kernels: vectors per lane (1, 2 or 4)
+  int chunks;     //   and workgroups per row = ceil(row_vecs / (BLOCK * nv))
+  int nvw;        // wave-per-row kernels: vectors per lane of the row's wave
+  int wchunks;    //   and chunks per row = ceil(row_vecs / (64 * nvw))
   int nle;
   int max_recv;
   uint32_t magic; // ceil(2^32 / nle)
@@ -636,6 +866,13 @@ void row_geometry(Geometry& g, int hidden_dim, bool ptrs_16B) {
   g.row_vecs = g.vec16 ? (int)(row_bytes / 16) : hidden_dim;
   g.nv = g.row_vecs <= BLOCK ? 1 : g.row_vecs <= 2 * BLOCK ? 2 : 4;
   g.chunks = (g.row_vecs + BLOCK * g.nv - 1) / (BLOCK * g.nv);
+  g.nvw = 16;
+  if (g.vec16) {
+    const int need = (g.row_vecs + 63) / 64;
+    for (int c : {14, 12, 8, 6, 4, 2, 1})
+      if (need <= c) g.nvw = c;
+  }
+  g.wchunks = (g.row_vecs + 64 * g.nvw - 1) / (64 * g.nvw);
 }
 
 template <typename... P>
@@ -674,6 +911,30 @@ int launch_status() { return hipGetLastError() == hipSuccess ? MOE_A2A_OK : MOE_
     }                                                      \
   } while (0)
 
+// Same for the wave-per-row kernels: <vector type, vectors per lane of a wave>.
+#define MOE_A2A_FOR_WAVE_KERNEL(G, LAUNCH)        \
+  do {                                            \
+    if ((G).vec16) {                              \
+      switch ((G).nvw) {                          \
+        case 1: LAUNCH(b128, 1); break;           \
+        case 2: LAUNCH(b128, 2); break;           \
+        case 4: LAUNCH(b128, 4); break;           \
+        case 6: LAUNCH(b128, 6); break;           \
+        case 8: LAUNCH(b128, 8); break;           \
+        case 12: LAUNCH(b128, 12); break;         \
+        case 14: LAUNCH(b128, 14); break;         \
+        default: LAUNCH(b128, 16); break;         \
+      }                                           \
+    } else {                                      \
+      LAUNCH(uint16_t, 16);                       \
+    }                                             \
+  } while (0)
+
+// Workgroups of a ranked row move over `rows` rows.
+long long group_items(long long rows, const Geometry& g) {
+  return (rows + ROWS - 1) / ROWS * g.wchunks;
+}
+
 }  // namespace
 
 extern "C" {
@@ -699,14 +960,14 @@ int moe_a2a_dispatch_send(const moe_a2a_shape* s, const void* x, const int32_t* 
   if (S > 0 && (!x || !indices || !send_buf || !send_meta)) return MOE_A2A_EINVAL;
   if (!all_aligned(2, x, send_buf)) return MOE_A2A_EALIGN;
   const Geometry g = geometry(s, x, send_buf);
-  if (!items_fit(S, g.chunks)) return MOE_A2A_EINVAL;
-  const int grid = s->world_size + mover_blocks(S * g.chunks);
+  if (!items_fit(S, g.wchunks)) return MOE_A2A_EINVAL;
+  const int grid = s->world_size + mover_blocks(group_items(S, g));
   hipStream_t st = (hipStream_t)stream;
-#define LAUNCH(V, NV)                                                                          \
-  dispatch_send_kernel<V, NV><<<grid, BLOCK, 0, st>>>(                                         \
+#define LAUNCH(V, NVW)                                                                         \
+  dispatch_send_kernel<V, NVW><<<grid, 64 * ROWS, 0, st>>>(                                    \
       (const V*)x, indices, (int)S, s->experts_per_token, g.nle, s->num_experts, s->world_size, \
-      g.magic, s->rank, g.row_vecs, g.chunks, (V*)send_buf, send_meta, send_counts, send_slot)
-  MOE_A2A_FOR_ROW_KERNEL(g, LAUNCH);
+      g.magic, s->rank, g.row_vecs, g.wchunks, (V*)send_buf, send_meta, send_counts, send_slot)
+  MOE_A2A_FOR_WAVE_KERNEL(g, LAUNCH);
 #undef LAUNCH
   return launch_status();
 }
@@ -722,14 +983,14 @@ int moe_a2a_dispatch_recv(const moe_a2a_shape* s, const void* recv_buf, const in
   if (!all_aligned(2, recv_buf, expert_x)) return MOE_A2A_EALIGN;
   const Geometry g = geometry(s, recv_buf, expert_x);
   // the stream can hold at most nle * max_recv rows that fit the expert buffers
-  if (!items_fit((long long)g.nle * g.max_recv, g.chunks)) return MOE_A2A_EINVAL;
-  const int grid = g.nle + mover_blocks((long long)rows_hint * g.chunks);
+  if (!items_fit((long long)g.nle * g.max_recv, g.wchunks)) return MOE_A2A_EINVAL;
+  const int grid = g.nle + mover_blocks(group_items(rows_hint, g));
   hipStream_t st = (hipStream_t)stream;
-#define LAUNCH(V, NV)                                                                       \
-  dispatch_recv_kernel<V, NV><<<grid, BLOCK, 0, st>>>(                                      \
+#define LAUNCH(V, NVW)                                                                      \
+  dispatch_recv_kernel<V, NVW><<<grid, 64 * ROWS, 0, st>>>(                                 \
       (const V*)recv_buf, recv_meta, recv_counts, s->world_size, g.nle, g.magic, g.max_recv, \
-      g.row_vecs, g.chunks, expert_num_tokens, (V*)expert_x, expert_meta)
-  MOE_A2A_FOR_ROW_KERNEL(g, LAUNCH);
+      g.row_vecs, g.wchunks, expert_num_tokens, (V*)expert_x, expert_meta)
+  MOE_A2A_FOR_WAVE_KERNEL(g, LAUNCH);
 #undef LAUNCH
   return launch_status();
 }
@@ -744,14 +1005,14 @@ int moe_a2a_combine_send(const moe_a2a_shape* s, const void* expert_y, const int
   if (!all_aligned(2, expert_y, send_buf)) return MOE_A2A_EALIGN;
   const Geometry g = geometry(s, expert_y, send_buf);
   if (g.nle > MAX_LOCAL_EXPERTS) return MOE_A2A_EINVAL;
-  if (!items_fit((long long)g.nle * g.max_recv, g.chunks)) return MOE_A2A_EINVAL;
-  const int grid = s->world_size + mover_blocks((long long)rows_hint * g.chunks);
+  if (!items_fit((long long)g.nle * g.max_recv, g.wchunks)) return MOE_A2A_EINVAL;
+  const int grid = s->world_size + mover_blocks(group_items(rows_hint, g));
   hipStream_t st = (hipStream_t)stream;
-#define LAUNCH(V, NV)                                                                         \
-  combine_send_kernel<V, NV><<<grid, BLOCK, 0, st>>>(                                         \
+#define LAUNCH(V, NVW)                                                                        \
+  combine_send_kernel<V, NVW><<<grid, 64 * ROWS, 0, st>>>(                                    \
       (const V*)expert_y, expert_meta, expert_num_tokens, g.nle, g.max_recv, s->world_size,    \
-      g.row_vecs, g.chunks, (V*)send_buf, send_meta, send_counts)
-  MOE_A2A_FOR_ROW_KERNEL(g, LAUNCH);
+      g.row_vecs, g.wchunks, (V*)send_buf, send_meta, send_counts)
+  MOE_A2A_FOR_WAVE_KERNEL(g, LAUNCH);
 #undef LAUNCH
   return launch_status();
 }
@@ -768,8 +1029,14 @@ int moe_a2a_combine_recv(const moe_a2a_shape* s, const void* recv_buf, const int
   const Geometry g = geometry(s, recv_buf, out_tokens);
   // wide rows: one 1024-lane workgroup per token scans the arrivals once; narrower rows use
   // 256 lanes with one or two vector columns each
-  const int blk = g.row_vecs >= 768 ? 1024 : BLOCK;
-  const int nv = blk == 1024 ? 1 : g.row_vecs <= BLOCK ? 1 : 2;
+#ifndef MOE_A2A_COMBINE_WIDE
+#define MOE_A2A_COMBINE_WIDE 1024
+#endif
+#ifndef MOE_A2A_COMBINE_NV
+#define MOE_A2A_COMBINE_NV 1
+#endif
+  const int blk = g.row_vecs >= 768 ? MOE_A2A_COMBINE_WIDE : BLOCK;
+  const int nv = g.row_vecs >= 768 ? MOE_A2A_COMBINE_NV : g.row_vecs <= BLOCK ? 1 : 2;
   const int chunks = (g.row_vecs + blk * nv - 1) / (blk * nv);
   if (!items_fit(num_tokens, chunks)) return MOE_A2A_EINVAL;
   const int grid = mover_blocks((long long)num_tokens * chunks);
@@ -782,6 +1049,7 @@ int moe_a2a_combine_recv(const moe_a2a_shape* s, const void* recv_buf, const int
 #define PICK_SHAPE(V, DT)                                  \
   do {                                                     \
     if (blk == 1024) { LAUNCH(V, DT, 1024, 1); }           \
+    else if (blk == 512) { LAUNCH(V, DT, 512, 1); }        \
     else if (nv == 1) { LAUNCH(V, DT, BLOCK, 1); }         \
     else { LAUNCH(V, DT, BLOCK, 2); }                      \
   } while (0)

@@ -234,3 +234,47 @@ def test_full_size_properties_without_oracle():
                     assert torch.equal(g["expert_x"][le, :n][sel], dev[s].x[tok])
                     assert bool((dev[s].indices[tok, kk] == r * nle + le).all())
     assert total == sum(d.num_tokens for d in dev) * K
+
+
+@pytest.mark.parametrize("name", ["bf16", "fp16"])
+def test_rounding_of_every_bit_pattern_through_combine_and_expert(name):
+    """All 65536 input bit patterns (infinities, NaNs, subnormals, ties included)
+    as addends, with weights that force roundings: the kernel's hardware
+    conversions must agree with the oracle's explicit round-to-nearest-even.
+    NaN results must be NaN; bf16 NaNs must be torch's canonical 0x7fc0."""
+    dt = DTYPES[name]
+    H, T, K = 2048, 32, 2
+    allbits = np.arange(65536, dtype=np.uint32).astype(np.uint16).reshape(T, H)
+    rng = np.random.default_rng(3)
+    second = orc.f32_to_b16(rng.standard_normal((T, H)).astype(np.float32) * 3, name)
+    cfg = MoEConfig(2, K, H, T, dt, dt)
+    a = LocalWorld(cfg, 1, device=DEV).ranks[0]
+    ret_buf = torch.cat([from_bits(allbits, dt), from_bits(second, dt)]).to(DEV)
+    meta = np.zeros((2 * T, 5), np.int32)
+    meta[:T, 2] = np.arange(T); meta[T:, 2] = np.arange(T); meta[T:, 3] = 1
+    w = (1 + rng.random((T, K), dtype=np.float32) * 2.0 ** -6).astype(np.float32)
+    w[::4, 0] = 1.0
+    counts = torch.tensor([2 * T], dtype=torch.int32, device=DEV)
+    y = torch.empty(T, H, dtype=dt, device=DEV)
+    a.combine_recv(y, torch.from_numpy(w).to(DEV), counts, ret_buf, torch.from_numpy(meta).to(DEV),
+                   accumulate=False)
+    torch.cuda.synchronize()
+    want = orc.combine_recv(np.concatenate([allbits, second]), meta, w, T, name)
+    got = bits(y)
+    nan = np.isnan(orc.b16_to_f32(want, name))
+    assert np.array_equal(got[~nan], want[~nan])
+    assert np.isnan(orc.b16_to_f32(got[nan], name)).all()
+    if name == "bf16":
+        assert (got[nan] == 0x7FC0).all()
+    # the simulated expert on the same patterns, rank 2 of 3 (scale 3)
+    cfg3 = MoEConfig(3, 1, H, T, dt, dt)
+    b = LocalWorld(cfg3, 3, device=DEV).ranks[2]
+    ex = torch.zeros(1, 3 * T, H, dtype=dt, device=DEV)
+    ex[0, :T] = from_bits(allbits, dt).to(DEV)
+    ey = b.expert_scale(ex, torch.tensor([T], dtype=torch.int32, device=DEV), T)
+    torch.cuda.synchronize()
+    want = orc.expert_scale(allbits, 2, name, name)
+    got = bits(ey[0, :T])
+    nan = np.isnan(orc.b16_to_f32(want, name))
+    assert np.array_equal(got[~nan], want[~nan])
+    assert np.isnan(orc.b16_to_f32(got[nan], name)).all()
