@@ -24,6 +24,7 @@
 #include <hip/hip_fp16.h>
 #include <stdint.h>
 #include <limits.h>
+#include <type_traits>
 
 #include "moe_a2a.h"
 
@@ -175,10 +176,14 @@ struct Payload {
   }
 };
 
+// Sum of max(counts[i], 0) over i < n, computed by every wave on its own: the
+// lanes load the counts side by side (one memory round trip instead of n
+// dependent scalar loads) and reduce with the wave butterfly.
 __device__ __forceinline__ int sum_counts(const int* __restrict__ counts, int n) {
+  const int lane = threadIdx.x & 63;
   int s = 0;
-  for (int i = 0; i < n; ++i) s += max(counts[i], 0);
-  return s;
+  for (int i = lane; i < n; i += 64) s += max(counts[i], 0);
+  return __builtin_amdgcn_readfirstlane(wave_sum(s));
 }
 
 // Number of keys i in [0, n) that pass `test(key_i, i)`, summed over the lanes
@@ -189,7 +194,9 @@ constexpr int SCAN_UNROLL = 8;
 template <int BLK, typename Keys, typename Test>
 __device__ __forceinline__ int count_keys(int n, const Keys& keys, Test test) {
   int cnt = 0;
-  for (int i = threadIdx.x; i < n; i += SCAN_UNROLL * BLK) {
+  // the trip count is the same for every lane: fetch() may use wave shuffles
+  for (int b = 0; b < n; b += SCAN_UNROLL * BLK) {
+    const int i = b + threadIdx.x;
     int idx[SCAN_UNROLL], key[SCAN_UNROLL];
 #pragma unroll
     for (int u = 0; u < SCAN_UNROLL; ++u) idx[u] = min(i + u * BLK, n - 1);
@@ -239,12 +246,15 @@ struct WavePayload {
 template <typename Keys>
 struct RowsScan {
   static constexpr int STEP = 64 * ROWS;
-  int n, i;
+  int n, b;  // number of keys; first key of the batch in flight (same for every lane)
   int key[SCAN_UNROLL];
-  __device__ __forceinline__ RowsScan(int n_, const Keys& keys) : n(n_), i(threadIdx.x) {
-    if (i < n) issue(keys);
+  __device__ __forceinline__ RowsScan(int n_, const Keys& keys) : n(n_), b(0) {
+    if (n > 0) issue(keys);
   }
+  // Every lane of the workgroup takes part (fetch() may use wave shuffles);
+  // lanes whose keys fall past n load key n-1 and are masked in consume().
   __device__ __forceinline__ void issue(const Keys& keys) {
+    const int i = b + threadIdx.x;
     int idx[SCAN_UNROLL];
 #pragma unroll
     for (int u = 0; u < SCAN_UNROLL; ++u) idx[u] = min(i + u * STEP, n - 1);
@@ -252,6 +262,7 @@ struct RowsScan {
   }
   template <typename Test>
   __device__ __forceinline__ void consume(Test test, int (&cnt)[ROWS]) const {
+    const int i = b + threadIdx.x;
 #pragma unroll
     for (int u = 0; u < SCAN_UNROLL; ++u) {
       const int i2 = i + u * STEP;
@@ -268,8 +279,8 @@ struct RowsScan {
   __device__ __forceinline__ void finish(const Keys& keys, Test test, int (&cnt)[ROWS]) {
 #pragma unroll
     for (int r = 0; r < ROWS; ++r) cnt[r] = 0;
-    if (i < n) consume(test, cnt);
-    for (i += SCAN_UNROLL * STEP; i < n; i += SCAN_UNROLL * STEP) {
+    if (n > 0) consume(test, cnt);
+    for (b += SCAN_UNROLL * STEP; b < n; b += SCAN_UNROLL * STEP) {
       issue(keys);
       consume(test, cnt);
     }
@@ -487,15 +498,71 @@ struct ExpertStreamKeys {
 #pragma unroll
     for (int u = 0; u < SCAN_UNROLL; ++u) le[u] = 0;
     for (int step = top; step > 0; step >>= 1) {
+      // all reads of a step first, then all updates: the reads stay in flight together
+      int c[SCAN_UNROLL], v[SCAN_UNROLL];
 #pragma unroll
-      for (int u = 0; u < SCAN_UNROLL; ++u) {
-        const int c = min(le[u] + step, nle);  // pre[nle] > g: never taken
-        le[u] = pre[c] <= g[u] ? c : le[u];
-      }
+      for (int u = 0; u < SCAN_UNROLL; ++u) c[u] = min(le[u] + step, nle);  // pre[nle] > g: never taken
+#pragma unroll
+      for (int u = 0; u < SCAN_UNROLL; ++u) v[u] = pre[c[u]];
+#pragma unroll
+      for (int u = 0; u < SCAN_UNROLL; ++u) le[u] = v[u] <= g[u] ? c[u] : le[u];
     }
+    int first[SCAN_UNROLL];
+#pragma unroll
+    for (int u = 0; u < SCAN_UNROLL; ++u) first[u] = pre[le[u]];
 #pragma unroll
     for (int u = 0; u < SCAN_UNROLL; ++u) {
-      const size_t row = (size_t)le[u] * max_recv + (g[u] - pre[le[u]]);
+      const size_t row = (size_t)le[u] * max_recv + (g[u] - first[u]);
+      key[u] = meta[row * META + FIELD];
+    }
+  }
+};
+
+// The same stream when there are at most 64 local experts: lane l of every wave
+// keeps the prefix of expert l in a register, so there is no LDS table, no
+// barrier and the row a wave owns is found with one ballot. Lanes at or past
+// nle hold the total, which no row index reaches.
+struct WaveExpertPrefix {
+  int excl, incl;  // rows before / up to and including expert `lane`
+  int total;
+  __device__ __forceinline__ WaveExpertPrefix(const int* __restrict__ cnt, int nle, int max_recv) {
+    const int lane = threadIdx.x & 63;
+    const int c = lane < nle ? min(max(cnt[lane], 0), max_recv) : 0;
+    incl = wave_inclusive_scan(c);
+    excl = incl - c;
+    total = __builtin_amdgcn_readlane(incl, 63);
+  }
+  // expert holding row g (wave-uniform g < total) and the number of rows before it
+  __device__ __forceinline__ void locate(int g, int& le, int& first) const {
+    le = __popcll(__ballot(incl <= g));
+    first = __builtin_amdgcn_readlane(excl, le);
+  }
+};
+
+template <int FIELD>
+struct WaveStreamKeys {
+  int excl;  // this lane's WaveExpertPrefix::excl
+  const int* __restrict__ meta;
+  int nle, top, max_recv;
+  __device__ __forceinline__ void fetch(const int* g, int* key) const {
+    int le[SCAN_UNROLL];
+#pragma unroll
+    for (int u = 0; u < SCAN_UNROLL; ++u) le[u] = 0;
+    for (int step = top; step > 0; step >>= 1) {
+      int c[SCAN_UNROLL], v[SCAN_UNROLL];
+#pragma unroll
+      for (int u = 0; u < SCAN_UNROLL; ++u) c[u] = le[u] + step;  // at most 32+16+...+1 = 63
+#pragma unroll
+      for (int u = 0; u < SCAN_UNROLL; ++u) v[u] = __shfl(excl, c[u], 64);
+#pragma unroll
+      for (int u = 0; u < SCAN_UNROLL; ++u) le[u] = v[u] <= g[u] ? c[u] : le[u];
+    }
+    int first[SCAN_UNROLL];
+#pragma unroll
+    for (int u = 0; u < SCAN_UNROLL; ++u) first[u] = __shfl(excl, le[u], 64);
+#pragma unroll
+    for (int u = 0; u < SCAN_UNROLL; ++u) {
+      const size_t row = (size_t)le[u] * max_recv + (g[u] - first[u]);
       key[u] = meta[row * META + FIELD];
     }
   }
@@ -508,7 +575,7 @@ struct ExpertStreamKeys {
 // order. Row g with origin d goes to slot
 //   #{rows of a lower origin} + #{earlier rows of origin d}.
 
-template <typename V, int NVW>
+template <typename V, int NVW, bool SMALL>
 __global__ __launch_bounds__(64 * ROWS) void combine_send_kernel(
     const V* __restrict__ expert_y, const int* __restrict__ expert_meta,
     const int* __restrict__ expert_num_tokens, int nle, int max_recv, int W, int row_vecs,
@@ -516,10 +583,21 @@ __global__ __launch_bounds__(64 * ROWS) void combine_send_kernel(
     int* __restrict__ send_counts) {
   __shared__ int part[ROWS * ROWS];
   __shared__ int s_d[ROWS];
-  __shared__ int pre[MAX_LOCAL_EXPERTS + 1];
+  __shared__ int pre[SMALL ? 1 : MAX_LOCAL_EXPERTS + 1];
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
-  const int R = expert_prefix<ROWS>(expert_num_tokens, nle, max_recv, pre, part);
-  const ExpertStreamKeys<1> key{pre, expert_meta, nle, top_step(nle), max_recv};
+
+  // SMALL (nle <= 64): prefix in registers; otherwise the LDS table
+  using Keys = typename std::conditional<SMALL, WaveStreamKeys<1>, ExpertStreamKeys<1>>::type;
+  int R, my_excl = 0, my_incl = 0;
+  if constexpr (SMALL) {
+    const WaveExpertPrefix wp(expert_num_tokens, nle, max_recv);
+    R = wp.total; my_excl = wp.excl; my_incl = wp.incl;
+  } else {
+    R = expert_prefix<ROWS>(expert_num_tokens, nle, max_recv, pre, part);
+  }
+  Keys key;
+  if constexpr (SMALL) key = Keys{my_excl, expert_meta, nle, 32, max_recv};
+  else key = Keys{pre, expert_meta, nle, top_step(nle), max_recv};
 
   if ((int)blockIdx.x < W) {
     const int me = blockIdx.x;
@@ -537,13 +615,20 @@ __global__ __launch_bounds__(64 * ROWS) void combine_send_kernel(
     const bool valid = g < R;
     const int gc = min(g, R - 1);
     const int base = c * (64 * NVW);
-    const int le = expert_of(pre, nle, key.top, gc);
-    const size_t row = (size_t)le * max_recv + (gc - pre[le]);
+    int le, first;
+    if constexpr (SMALL) {
+      le = __popcll(__ballot(my_incl <= gc));
+      first = __builtin_amdgcn_readlane(my_excl, le);
+    } else {
+      le = expert_of(pre, nle, key.top, gc);
+      first = pre[le];
+    }
+    const size_t row = (size_t)le * max_recv + (gc - first);
 
     int m = 0;
     if (c == 0 && lane < META) m = expert_meta[row * META + lane];
     const int d = expert_meta[row * META + 1];
-    RowsScan<ExpertStreamKeys<1>> scan(R, key);
+    RowsScan<Keys> scan(R, key);
     WavePayload<V, NVW> p;
     p.load(expert_y + row * row_vecs, base, row_vecs, lane);
 
@@ -1008,12 +1093,18 @@ int moe_a2a_combine_send(const moe_a2a_shape* s, const void* expert_y, const int
   if (!items_fit((long long)g.nle * g.max_recv, g.wchunks)) return MOE_A2A_EINVAL;
   const int grid = s->world_size + mover_blocks(group_items(rows_hint, g));
   hipStream_t st = (hipStream_t)stream;
-#define LAUNCH(V, NVW)                                                                        \
-  combine_send_kernel<V, NVW><<<grid, 64 * ROWS, 0, st>>>(                                    \
+#define LAUNCH_S(V, NVW, SMALL)                                                                \
+  combine_send_kernel<V, NVW, SMALL><<<grid, 64 * ROWS, 0, st>>>(                             \
       (const V*)expert_y, expert_meta, expert_num_tokens, g.nle, g.max_recv, s->world_size,    \
       g.row_vecs, g.wchunks, (V*)send_buf, send_meta, send_counts)
+#define LAUNCH(V, NVW)                        \
+  do {                                        \
+    if (g.nle <= 64) LAUNCH_S(V, NVW, true);  \
+    else LAUNCH_S(V, NVW, false);             \
+  } while (0)
   MOE_A2A_FOR_WAVE_KERNEL(g, LAUNCH);
 #undef LAUNCH
+#undef LAUNCH_S
   return launch_status();
 }
 
@@ -1030,7 +1121,7 @@ int moe_a2a_combine_recv(const moe_a2a_shape* s, const void* recv_buf, const int
   // wide rows: one 1024-lane workgroup per token scans the arrivals once; narrower rows use
   // 256 lanes with one or two vector columns each
 #ifndef MOE_A2A_COMBINE_WIDE
-#define MOE_A2A_COMBINE_WIDE 1024
+#define MOE_A2A_COMBINE_WIDE 256
 #endif
 #ifndef MOE_A2A_COMBINE_NV
 #define MOE_A2A_COMBINE_NV 1
