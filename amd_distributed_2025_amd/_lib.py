@@ -7,8 +7,11 @@ from __future__ import annotations
 import ctypes as C
 from pathlib import Path
 
+import os
+
 PKG_DIR = Path(__file__).resolve().parent
-LIBRARY = PKG_DIR / "libmoe_a2a.so"
+# MOE_A2A_LIBRARY points at another build of the same ABI (used to compare tuning variants)
+LIBRARY = Path(os.environ.get("MOE_A2A_LIBRARY") or PKG_DIR / "libmoe_a2a.so")
 
 F16, BF16 = 0, 1
 

@@ -48,21 +48,31 @@ constexpr int NUM_XCD = 8;
 // struct whose copies become memcpy calls that can pin a local in memory.)
 typedef unsigned int b128 __attribute__((ext_vector_type(4)));
 
-// Row payload is written once and read by a later kernel, never by this one:
-// streaming (nontemporal) stores keep it from write-allocating in L2.
-#ifndef MOE_A2A_NT_STORE
-#define MOE_A2A_NT_STORE 1
+// Streaming (nontemporal) stores do not write-allocate in L2, which makes the
+// writing kernel about a quarter faster, but a kernel that reads the rows right
+// afterwards then fetches them from HBM and loses more than the writer gained.
+// So they are used only for the two buffers whose next reader is the exchange
+// (in a multi-GPU job: the fabric), not for expert_x / expert_y, which the
+// expert computation reads next on the same device.
+#ifndef MOE_A2A_NT_SEND   /* stage 1 -> send buffer */
+#define MOE_A2A_NT_SEND 1
+#endif
+#ifndef MOE_A2A_NT_RECV   /* stage 2 -> expert_x */
+#define MOE_A2A_NT_RECV 0
+#endif
+#ifndef MOE_A2A_NT_CSEND  /* stage 3 -> send-back buffer */
+#define MOE_A2A_NT_CSEND 1
+#endif
+#ifndef MOE_A2A_NT_STANDIN /* expert and exchange stand-ins */
+#define MOE_A2A_NT_STANDIN 0
 #endif
 #ifndef MOE_A2A_NT_LOAD
 #define MOE_A2A_NT_LOAD 0
 #endif
-template <typename V>
-__device__ __forceinline__ void stream_store(V* p, const V& v) {
-#if MOE_A2A_NT_STORE
-  __builtin_nontemporal_store(v, p);
-#else
-  *p = v;
-#endif
+template <bool NT, typename V>
+__device__ __forceinline__ void row_store(V* p, const V& v) {
+  if constexpr (NT) __builtin_nontemporal_store(v, p);
+  else *p = v;
 }
 template <typename V>
 __device__ __forceinline__ V stream_load(const V* p) {
@@ -83,10 +93,31 @@ __device__ __forceinline__ void lds_barrier() {
   asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
 }
 
-__device__ __forceinline__ int wave_sum(int v) {
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+// Inclusive prefix sum across the 64 lanes of a wave, in the VALU's
+// data-parallel-primitive (DPP) lane network: four row_shr steps scan each row
+// of 16 lanes, row_bcast15 / row_bcast31 carry the row totals across rows.
+// Six dependent VALU ops; a __shfl-based scan would take six round trips through
+// the LDS crossbar, which is what dominates a slot computation of a few hundred
+// cycles.
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ int dpp_add(int v) {
+  // lanes whose source lies outside the row, or whose row is masked off, add 0
+  return v + __builtin_amdgcn_update_dpp(0, v, CTRL, ROW_MASK, 0xf, false);
+}
+
+__device__ __forceinline__ int wave_inclusive_scan(int v) {
+  v = dpp_add<0x111, 0xf>(v);  // row_shr:1
+  v = dpp_add<0x112, 0xf>(v);  // row_shr:2
+  v = dpp_add<0x114, 0xf>(v);  // row_shr:4
+  v = dpp_add<0x118, 0xf>(v);  // row_shr:8
+  v = dpp_add<0x142, 0xa>(v);  // row_bcast15 into rows 1 and 3
+  v = dpp_add<0x143, 0xc>(v);  // row_bcast31 into rows 2 and 3
   return v;
+}
+
+// Sum over the wave, returned to every lane.
+__device__ __forceinline__ int wave_sum(int v) {
+  return __builtin_amdgcn_readlane(wave_inclusive_scan(v), 63);
 }
 
 // Sum over a workgroup of NW waves; every lane gets the total. `red` is NW ints
@@ -102,17 +133,6 @@ __device__ __forceinline__ int block_sum(int v, int* red) {
   for (int w = 0; w < NW; ++w) s += red[w];
   lds_barrier();
   return s;
-}
-
-// Inclusive prefix sum across the 64 lanes of a wave.
-__device__ __forceinline__ int wave_inclusive_scan(int v) {
-  const int lane = threadIdx.x & 63;
-#pragma unroll
-  for (int o = 1; o < 64; o <<= 1) {
-    int n = __shfl_up(v, o, 64);
-    if (lane >= o) v += n;
-  }
-  return v;
 }
 
 // Workgroups are handed to the 8 XCDs round-robin by blockIdx. This bijection
@@ -166,7 +186,7 @@ struct Payload {
 #pragma unroll
     for (int j = 0; j < NV; ++j) {
       const int idx = base + j * BLOCK + threadIdx.x;
-      if (idx < row_vecs) stream_store(row + idx, v[j]);
+      if (idx < row_vecs) row_store<(MOE_A2A_NT_STANDIN != 0)>(row + idx, v[j]);
     }
   }
   template <typename F>
@@ -228,11 +248,12 @@ struct WavePayload {
 #pragma unroll
     for (int j = 0; j < NVW; ++j) v[j] = stream_load(row + min(base + j * 64 + lane, row_vecs - 1));
   }
+  template <bool NT>
   __device__ __forceinline__ void store(V* __restrict__ row, int base, int row_vecs, int lane) const {
 #pragma unroll
     for (int j = 0; j < NVW; ++j) {
       const int idx = base + j * 64 + lane;
-      if (idx < row_vecs) stream_store(row + idx, v[j]);
+      if (idx < row_vecs) row_store<NT>(row + idx, v[j]);
     }
   }
 };
@@ -359,7 +380,7 @@ __global__ __launch_bounds__(64 * ROWS) void dispatch_send_kernel(
     const int slot = rows_reduce(cnt, part, wave, lane);
 
     if (valid) {
-      p.store(send_buf + (size_t)slot * row_vecs, base, row_vecs, lane);
+      p.template store<(MOE_A2A_NT_SEND != 0)>(send_buf + (size_t)slot * row_vecs, base, row_vecs, lane);
       if (c == 0) {
         if (lane < META) {
           int m = lane == 0 ? e : lane == 1 ? rank : lane == 2 ? t : lane == 3 ? k : 0;
@@ -429,7 +450,7 @@ __global__ __launch_bounds__(64 * ROWS) void dispatch_recv_kernel(
 
     if (valid && pos < max_recv) {
       const size_t row = (size_t)le * max_recv + pos;
-      p.store(expert_x + row * row_vecs, base, row_vecs, lane);
+      p.template store<(MOE_A2A_NT_RECV != 0)>(expert_x + row * row_vecs, base, row_vecs, lane);
       if (c == 0 && lane < META) expert_meta[row * META + lane] = m;
     }
   }
@@ -645,7 +666,7 @@ __global__ __launch_bounds__(64 * ROWS) void combine_send_kernel(
     const int slot = rows_reduce(cnt, part, wave, lane);
 
     if (valid) {
-      p.store(send_buf + (size_t)slot * row_vecs, base, row_vecs, lane);
+      p.template store<(MOE_A2A_NT_CSEND != 0)>(send_buf + (size_t)slot * row_vecs, base, row_vecs, lane);
       if (c == 0 && lane < META) send_meta[(size_t)slot * META + lane] = m;
     }
   }

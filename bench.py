@@ -15,10 +15,10 @@ once, before timing, by running the peers' own kernels on their seeded inputs;
 they stay resident where an exchange would have written them.
 
 Prints ONE JSON line. `value` is the wall time of a whole step (stand-ins
-included) in microseconds; `hot_path_us` is the sum of the four path kernels
-alone, each timed with HIP events on the launch stream; `roofline` prices the
-slowest of those four against HBM peak with the algorithmic bytes of that
-stage; `cpu_baseline` is the row-by-row torch-CPU statement of the same step
+included) in microseconds; `hot_path_us` is the sum of the four path kernels,
+each timed in place (HIP events on the launch stream around graphs of whole
+steps with and without that kernel); `roofline` prices the slowest of those
+four against HBM peak with the algorithmic bytes of that stage; `cpu_baseline` is the row-by-row torch-CPU statement of the same step
 timed on this box's host cores.
 """
 from __future__ import annotations
@@ -48,7 +48,8 @@ def parse_args():
     ap.add_argument("--seed", type=int, default=2025)
     ap.add_argument("--mode", default="graph", choices=["graph", "eager"],
                     help="replay a captured HIP graph of the step (default) or launch eagerly")
-    ap.add_argument("--kernel-reps", type=int, default=50, help="launches per kernel for the per-kernel timing")
+    ap.add_argument("--kernel-reps", type=int, default=20,
+                    help="whole steps per graph in the per-kernel (leave-one-out) timing")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="target CPU time of the cpu_baseline sample")
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
     return ap.parse_args()
@@ -163,35 +164,47 @@ def main():
     y_after = y[:T].clone()
     same_as_setup = bool(torch.equal(y_after, ys0[0]))
 
-    # ---- per-kernel timing: HIP events on the launch stream around back-to-back launches
-    def time_kernel(fn, reps):
-        # `reps` launches captured in one HIP graph, so the host's launch cost is not in the figure
+    # ---- per-kernel timing, in the pipeline: HIP events on the launch stream around a graph of
+    # `reps` whole steps, with and without the kernel. The difference is what the kernel costs where
+    # it runs, with its inputs in the cache state the previous kernel left them in (its launch gap
+    # included). A kernel timed alone in a loop re-reads inputs that nothing rewrote and looks faster.
+    def graph_of(fns, reps):
         side = torch.cuda.Stream()
         side.wait_stream(torch.cuda.current_stream())
         with torch.cuda.stream(side):
-            fn()
+            for fn in fns:
+                fn()
         torch.cuda.current_stream().wait_stream(side)
         torch.cuda.synchronize()
         gr = torch.cuda.CUDAGraph()
         with torch.cuda.graph(gr):
             for _ in range(reps):
-                fn()
+                for fn in fns:
+                    fn()
         gr.replay()
         torch.cuda.synchronize()
+        return gr
+
+    def time_graph(gr, reps, rounds=9):
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         samples = []
-        for _ in range(7):
+        for _ in range(rounds):
             e0.record()
             gr.replay()
             e1.record()
             e1.synchronize()
             samples.append(e0.elapsed_time(e1) * 1e3 / reps)
-        return statistics.median(samples), min(samples)
+        return statistics.median(samples)
 
+    reps = args.kernel_reps
+    full_us = time_graph(graph_of([fn for _, fn in stages], reps), reps)
     kern = {}
     for name, fn in stages:
-        med, best = time_kernel(fn, args.kernel_reps)
-        kern[name] = {"us": round(med, 3), "us_min": round(best, 3)}
+        without = time_graph(graph_of([f for n, f in stages if n != name], reps), reps)
+        alone = time_graph(graph_of([fn], reps), reps)
+        kern[name] = {"us": round(full_us - without, 3), "us_alone_warm": round(alone, 3)}
+    step()  # leave every buffer as a full step leaves it
+    torch.cuda.synchronize()
     ab = alg_bytes(T, K, H, R)
     for name in path:
         kern[name]["alg_bytes"] = ab[name]

@@ -1,0 +1,127 @@
+"""CPU-side checks: the C ABI library loads and exports what include/moe_a2a.h
+declares, argument errors are reported before anything is launched, and the
+host layer (input generator, shape checks, loud failure without a GPU) behaves."""
+import ctypes as C
+import re
+from pathlib import Path
+
+import numpy as np
+import pytest
+import torch
+
+from amd_distributed_2025_amd import _lib
+from amd_distributed_2025_amd.task import (TASK_YML_BENCHMARKS, TASK_YML_TESTS, WORKLOADS, MoEConfig,
+                                           generate_input, generate_world)
+
+ROOT = Path(__file__).resolve().parent.parent
+HEADER = (ROOT / "include" / "moe_a2a.h").read_text()
+
+
+def declared_functions():
+    names = re.findall(r"^(?:int|const char\*)\s+(moe_a2a_\w+)\s*\(", HEADER, flags=re.M)
+    assert len(names) >= 8
+    return names
+
+
+def test_library_exports_every_declared_symbol():
+    lib = _lib.load()
+    for name in declared_functions():
+        assert hasattr(lib, name), name
+    bound = set(_lib.SIGNATURES) | set(_lib.STRING_FUNCTIONS)
+    assert bound == set(declared_functions())
+    assert lib.moe_a2a_version().decode().startswith("moe_a2a")
+
+
+def test_argument_counts_match_the_header():
+    """ctypes signatures and header prototypes must list the same number of parameters."""
+    flat = re.sub(r"/\*.*?\*/", "", HEADER, flags=re.S)
+    for name, args in {**_lib.SIGNATURES, **_lib.STRING_FUNCTIONS}.items():
+        proto = re.search(name + r"\s*\((.*?)\);", flat, flags=re.S).group(1)
+        n = 0 if proto.strip() == "void" else proto.count(",") + 1
+        assert n == len(args), (name, n, len(args))
+
+
+def test_shape_struct_layout_matches_header():
+    fields = re.search(r"typedef struct moe_a2a_shape \{(.*?)\} moe_a2a_shape;", HEADER, flags=re.S).group(1)
+    names = re.findall(r"int32_t\s+(\w+);", fields)
+    assert names == [f[0] for f in _lib.Shape._fields_]
+    assert C.sizeof(_lib.Shape) == 4 * len(names)
+
+
+def test_bad_arguments_are_rejected_without_touching_the_gpu():
+    lib = _lib.load()
+    ok = _lib.Shape(8, 0, 256, 8, 7168, 256)
+    assert lib.moe_a2a_strerror(0) == b"ok"
+    for status in (-1, -2, -3, -99):
+        assert lib.moe_a2a_strerror(status)
+    one = C.c_void_p(16)  # never dereferenced: every call below fails validation first
+    # null shape / bad shapes
+    assert lib.moe_a2a_dispatch_send(None, one, one, 1, one, one, one, None, None) == -1
+    for bad in (_lib.Shape(0, 0, 8, 2, 16, 4), _lib.Shape(8, 8, 8, 2, 16, 4), _lib.Shape(8, 0, 12, 2, 16, 4),
+                _lib.Shape(8, 0, 8, 0, 16, 4), _lib.Shape(8, 0, 8, 2, 0, 4), _lib.Shape(1, 0, 1 << 17, 2, 16, 4)):
+        assert lib.moe_a2a_dispatch_send(C.byref(bad), one, one, 1, one, one, one, None, None) == -1
+    # token count beyond capacity, null buffers, odd alignment, bad dtype, bad ranks
+    assert lib.moe_a2a_dispatch_send(C.byref(ok), one, one, 257, one, one, one, None, None) == -1
+    assert lib.moe_a2a_dispatch_send(C.byref(ok), None, one, 4, one, one, one, None, None) == -1
+    assert lib.moe_a2a_dispatch_send(C.byref(ok), C.c_void_p(17), one, 4, one, one, one, None, None) == -2
+    assert lib.moe_a2a_dispatch_recv(C.byref(ok), one, one, None, 4, one, one, one, None) == -1
+    assert lib.moe_a2a_combine_send(C.byref(ok), one, one, one, -1, one, one, one, None) == -1
+    assert lib.moe_a2a_combine_recv(C.byref(ok), one, one, one, one, 4, one, 0, 7, None) == -1
+    assert lib.moe_a2a_expert_scale(C.byref(ok), one, one, 4, 0, 5, one, None) == -1
+    assert lib.moe_a2a_exchange_local(8, 16, one, one, one, 8, one, one, one, 0, 4, None) == -1
+    assert lib.moe_a2a_exchange_local(8, 16, one, one, one, 0, one, one, one, 0, 0, None) == 0  # nothing to move
+    with pytest.raises(_lib.MoeA2AError, match="invalid argument"):
+        _lib.call("moe_a2a_dispatch_send", None, one, one, 1, one, one, one, None, None)
+
+
+def test_no_silent_cpu_fallback():
+    from amd_distributed_2025_amd import HIPAllToAll, custom_kernel
+
+    cfg = MoEConfig(8, 2, 16, 4)
+    with pytest.raises(_lib.MoeA2AError):
+        HIPAllToAll(cfg, 0, 1, device="cpu")
+    data = generate_input(8, 2, 16, 4, seed=1, rank=0, world_size=1)
+    with pytest.raises(RuntimeError, match="GPU"):
+        custom_kernel(data)
+
+
+def test_product_never_imports_the_oracle():
+    for path in (ROOT / "amd_distributed_2025_amd").rglob("*.py"):
+        text = path.read_text()
+        assert "oracle" not in re.sub(r"#.*", "", text), path
+    assert "oracle" not in (ROOT / "amd_distributed_2025_amd" / "csrc" / "moe_a2a.hip").read_text()
+
+
+def test_generate_input_follows_the_reference_contract():
+    cfg, data, rank, world = generate_input(64, 6, 2048, 32, seed=7, rank=3, world_size=8)
+    assert (rank, world) == (3, 8) and cfg.in_dtype == torch.float16 == cfg.out_dtype
+    T = data.num_tokens
+    assert 1 <= T <= 31  # randint(1, max): upper end exclusive
+    assert data.indices.shape == (T, 6) and data.indices.dtype == torch.int32
+    assert data.weights.shape == (T, 6) and data.weights.dtype == torch.float32
+    assert data.x.shape == (T, 2048) and data.x.dtype == torch.float16
+    assert bool((data.weights >= 0).all()) and bool((data.weights < 1).all())
+    idx = data.indices.numpy()
+    assert idx.min() >= 0 and idx.max() < 64
+    assert all(len(set(r)) == 6 for r in idx.tolist())
+    # same seed, same data; another rank, other data
+    again = generate_input(64, 6, 2048, 32, seed=7, rank=3, world_size=8)[1]
+    assert torch.equal(again.x, data.x) and torch.equal(again.indices, data.indices)
+    other = generate_input(64, 6, 2048, 32, seed=7, rank=4, world_size=8)[1]
+    assert other.num_tokens != T or not torch.equal(other.indices, data.indices)
+
+
+def test_workload_generators():
+    w = generate_world(WORKLOADS["C4"], 1)
+    assert len(w) == 8 and all(d.num_tokens == 256 and d.x.dtype == torch.bfloat16 for _, d, _, _ in w)
+    assert np.allclose(w[0][1].weights.sum(1).numpy(), 1.0, atol=1e-5)  # softmax weights
+    skew = generate_world(WORKLOADS["C5"], 1)
+    ids = np.concatenate([d.indices.numpy().ravel() for _, d, _, _ in skew])
+    hist = np.sort(np.bincount(ids, minlength=256))[::-1]
+    assert hist[0] > 8 * hist[64]  # Zipf: the head expert is far hotter than the 65th
+    assert all(len(set(r)) == 8 for _, d, _, _ in skew for r in d.indices.tolist())
+    # all ranks of one job share the popularity ranking
+    hot0 = np.bincount(skew[0][1].indices.numpy().ravel(), minlength=256).argmax()
+    hot5 = np.bincount(skew[5][1].indices.numpy().ravel(), minlength=256).argmax()
+    assert hot0 == hot5 == np.bincount(ids, minlength=256).argmax()
+    assert len(TASK_YML_TESTS) == 9 and len(TASK_YML_BENCHMARKS) == 5
