@@ -123,7 +123,7 @@ class HIPAllToAll:
         _need(recv_counts, torch.int32, self.device, "recv_counts")
         _need(recv_buf, cfg.in_dtype, self.device, "recv_buf")
         _need(recv_meta, torch.int32, self.device, "recv_meta")
-        hint = min(recv_buf.shape[0], self.max_rows_in if rows_hint is None else rows_hint)
+        hint = min(recv_buf.shape[0], recv_meta.shape[0], self.max_rows_in if rows_hint is None else rows_hint)
         nle = self.num_local_experts
         num = self._buf("expert_num_tokens", (nle,), torch.int32)
         ex = self._buf("expert_x", (nle, self.max_recv, cfg.hidden_dim), cfg.in_dtype)
@@ -177,8 +177,9 @@ class HIPAllToAll:
         T = weights.shape[0]
         if out_tokens.shape[0] < T or out_tokens.shape[1] != cfg.hidden_dim:
             raise ValueError("combine: out_tokens must hold num_tokens rows of hidden_dim")
+        hint = min(ret_buf.shape[0], ret_meta.shape[0], T * cfg.experts_per_token)
         _lib.call("moe_a2a_combine_recv", self._shape_ref, _ptr(ret_buf), _ptr(ret_meta),
-                  _ptr(ret_counts), _ptr(weights), T, _ptr(out_tokens), int(bool(accumulate)),
+                  _ptr(ret_counts), hint, _ptr(weights), T, _ptr(out_tokens), int(bool(accumulate)),
                   _DT[dtype_name(cfg.out_dtype)], _stream(self.device))
         return out_tokens
 

@@ -267,9 +267,10 @@ struct WavePayload {
 template <typename Keys>
 struct RowsScan {
   static constexpr int STEP = 64 * ROWS;
-  int n, b;  // number of keys; first key of the batch in flight (same for every lane)
+  int n, b;  // keys that may be loaded; first key of the batch in flight (same for every lane)
   int key[SCAN_UNROLL];
-  __device__ __forceinline__ RowsScan(int n_, const Keys& keys) : n(n_), b(0) {
+  // `n_load` keys are known to be readable; how many of them count is told to finish().
+  __device__ __forceinline__ RowsScan(int n_load, const Keys& keys) : n(n_load), b(0) {
     if (n > 0) issue(keys);
   }
   // Every lane of the workgroup takes part (fetch() may use wave shuffles);
@@ -293,14 +294,17 @@ struct RowsScan {
       }
     }
   }
-  // The first batch is consumed in straight-line code, apart from the loop over
-  // later batches: inside a loop the compiler must assume the keys were the last
-  // loads issued and would wait for the payload as well.
+  // Counts over keys [0, n_valid), n_valid <= n_load. The first batch is consumed
+  // in straight-line code, apart from the loop over later batches: inside a loop
+  // the compiler must assume the keys were the last loads issued and would wait
+  // for the payload as well.
   template <typename Test>
-  __device__ __forceinline__ void finish(const Keys& keys, Test test, int (&cnt)[ROWS]) {
+  __device__ __forceinline__ void finish(const Keys& keys, int n_valid, Test test, int (&cnt)[ROWS]) {
 #pragma unroll
     for (int r = 0; r < ROWS; ++r) cnt[r] = 0;
-    if (n > 0) consume(test, cnt);
+    const bool first = n > 0;
+    n = min(n, n_valid);
+    if (first) consume(test, cnt);
     for (b += SCAN_UNROLL * STEP; b < n; b += SCAN_UNROLL * STEP) {
       issue(keys);
       consume(test, cnt);
@@ -310,19 +314,22 @@ struct RowsScan {
 
 // Total of cnt[wave] over the workgroup, returned to the lanes of that wave:
 // wave w gets the count that belongs to the group's row w. `part` is
-// ROWS*ROWS ints of LDS, reusable after the call.
-__device__ __forceinline__ int rows_reduce(const int (&cnt)[ROWS], int* part, int wave, int lane) {
+// 2*ROWS*ROWS ints of LDS used in halves by alternate calls (`parity` flips per
+// call), so one barrier per call is enough: a wave can only overwrite a half
+// after every wave has passed the barrier of the call in between.
+__device__ __forceinline__ int rows_reduce(const int (&cnt)[ROWS], int* part, int parity, int wave,
+                                           int lane) {
   if (ROWS == 1) return wave_sum(cnt[0]);
+  int* half = part + (parity & 1) * (ROWS * ROWS);
 #pragma unroll
   for (int r = 0; r < ROWS; ++r) {
     const int s = wave_sum(cnt[r]);
-    if (lane == 0) part[wave * ROWS + r] = s;
+    if (lane == 0) half[wave * ROWS + r] = s;
   }
   lds_barrier();
   int mine = 0;
 #pragma unroll
-  for (int w = 0; w < ROWS; ++w) mine += part[w * ROWS + wave];
-  lds_barrier();
+  for (int w = 0; w < ROWS; ++w) mine += half[w * ROWS + wave];
   return mine;
 }
 
@@ -337,8 +344,7 @@ __global__ __launch_bounds__(64 * ROWS) void dispatch_send_kernel(
     const V* __restrict__ x, const int* __restrict__ indices, int S, int K, int nle, int E, int W,
     uint32_t magic, int rank, int row_vecs, int chunks, V* __restrict__ send_buf,
     int* __restrict__ send_meta, int* __restrict__ send_counts, int* __restrict__ send_slot) {
-  __shared__ int part[ROWS * ROWS];
-  __shared__ int s_lo[ROWS], s_hi[ROWS];
+  __shared__ int part[2 * ROWS * ROWS];
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const StridedKeys key{indices, 1};
 
@@ -352,32 +358,36 @@ __global__ __launch_bounds__(64 * ROWS) void dispatch_send_kernel(
 
   const int groups = (S + ROWS - 1) / ROWS;
   const int items = groups * chunks, movers = gridDim.x - W;
-  for (int q = xcd_contiguous(blockIdx.x - W, movers); q < items; q += movers) {
+  int parity = 0;
+  for (int q = xcd_contiguous(blockIdx.x - W, movers); q < items; q += movers, ++parity) {
     const int grp = chunks == 1 ? q : q / chunks, c = q - grp * chunks;
-    const int i = grp * ROWS + wave;
+    const int i0 = grp * ROWS, i = i0 + wave;
     const bool valid = i < S;
-    const int ic = min(i, S - 1);
-    const int e = indices[ic];
-    const int t = ic / K, k = ic - t * K;
     const int base = c * (64 * NVW);
 
+    // every wave reads the expert ids of all rows of the group (the same few
+    // words for every lane), so no exchange between the waves is needed
+    int re[ROWS];
+#pragma unroll
+    for (int r = 0; r < ROWS; ++r) re[r] = indices[min(i0 + r, S - 1)];
     RowsScan<StridedKeys> scan(S, key);
+    const int ic = min(i, S - 1);
+    const int t = ic / K, k = ic - t * K;
     WavePayload<V, NVW> p;
     p.load(x + (size_t)t * row_vecs, base, row_vecs, lane);
 
-    int lo, hi, d;
-    dest_class(e, nle, E, magic, lo, hi, d);
-    if (lane == 0) { s_lo[wave] = lo; s_hi[wave] = hi; }
-    lds_barrier();
-    int rlo[ROWS], rhi[ROWS];
+    int rlo[ROWS], rhi[ROWS], e = 0;
 #pragma unroll
-    for (int r = 0; r < ROWS; ++r) { rlo[r] = s_lo[r]; rhi[r] = s_hi[r]; }
-    const int i0 = grp * ROWS;
+    for (int r = 0; r < ROWS; ++r) {
+      int d;
+      dest_class(re[r], nle, E, magic, rlo[r], rhi[r], d);
+      if (r == wave) e = re[r];
+    }
     int cnt[ROWS];
-    scan.finish(key, [&](int r, int e2, int i2) {
+    scan.finish(key, S, [&](int r, int e2, int i2) {
       return (e2 < rlo[r]) | ((e2 <= rhi[r]) & (e2 >= rlo[r]) & (i2 < i0 + r));
     }, cnt);
-    const int slot = rows_reduce(cnt, part, wave, lane);
+    const int slot = rows_reduce(cnt, part, parity, wave, lane);
 
     if (valid) {
       p.template store<(MOE_A2A_NT_SEND != 0)>(send_buf + (size_t)slot * row_vecs, base, row_vecs, lane);
@@ -397,20 +407,24 @@ __global__ __launch_bounds__(64 * ROWS) void dispatch_send_kernel(
 // grid = nle counting workgroups (rows per local expert) followed by one
 // workgroup per (group of ROWS received rows, chunk). Row i goes to expert
 // le = e % nle at position #{earlier rows of the same expert}.
+//
+// `hint_rows` rows of recv_buf / recv_meta are readable whatever the counts
+// say. A workgroup whose rows lie below that bound issues all its loads before
+// it knows the true row count R (the counts are loaded at the same time) and
+// only the stores wait for R; rows at or past R are loaded and dropped.
 
 template <typename V, int NVW>
 __global__ __launch_bounds__(64 * ROWS) void dispatch_recv_kernel(
     const V* __restrict__ recv_buf, const int* __restrict__ recv_meta,
-    const int* __restrict__ recv_counts, int W, int nle, uint32_t magic, int max_recv,
-    int row_vecs, int chunks, int* __restrict__ expert_num_tokens, V* __restrict__ expert_x,
-    int* __restrict__ expert_meta) {
-  __shared__ int part[ROWS * ROWS];
-  __shared__ int s_le[ROWS];
+    const int* __restrict__ recv_counts, int W, int hint_rows, int nle, uint32_t magic,
+    int max_recv, int row_vecs, int chunks, int* __restrict__ expert_num_tokens,
+    V* __restrict__ expert_x, int* __restrict__ expert_meta) {
+  __shared__ int part[2 * ROWS * ROWS];
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
-  const int R = sum_counts(recv_counts, W);
   const StridedKeys key{recv_meta, META};
 
   if ((int)blockIdx.x < nle) {
+    const int R = sum_counts(recv_counts, W);
     const int me = blockIdx.x;
     int c = count_keys<64 * ROWS>(R, key, [=](int e, int) { return floormod(e, nle, magic) == me; });
     c = block_sum<ROWS>(c, part);
@@ -418,42 +432,60 @@ __global__ __launch_bounds__(64 * ROWS) void dispatch_recv_kernel(
     return;
   }
 
-  const int groups = (R + ROWS - 1) / ROWS;
-  const int items = groups * chunks, movers = gridDim.x - nle;
-  for (int q = blockIdx.x - nle; q < items; q += movers) {
+  const int movers = gridDim.x - nle;
+  int parity = 0;
+  // One (group, chunk) item. `limit` rows may be read; R is evaluated after the
+  // loads are issued (it is already known on every pass but the first).
+  auto move = [&](int q, int limit, auto&& rows_known) {
     const int grp = chunks == 1 ? q : q / chunks, c = q - grp * chunks;
-    const int i = grp * ROWS + wave;
-    const bool valid = i < R;
-    const int ic = min(i, R - 1);
+    const int i0 = grp * ROWS, i = i0 + wave;
+    const int ic = min(i, limit - 1);
     const int base = c * (64 * NVW);
 
-    const int i0 = grp * ROWS;
+    int re[ROWS];
+#pragma unroll
+    for (int r = 0; r < ROWS; ++r) re[r] = recv_meta[(size_t)min(i0 + r, limit - 1) * META];
     int m = 0;
     if (c == 0 && lane < META) m = recv_meta[(size_t)ic * META + lane];
-    const int e = recv_meta[(size_t)ic * META];
     // only rows before the group's last row can precede any of its rows
-    RowsScan<StridedKeys> scan(min(i0 + ROWS - 1, R), key);
+    RowsScan<StridedKeys> scan(min(i0 + ROWS - 1, limit), key);
     WavePayload<V, NVW> p;
     p.load(recv_buf + (size_t)ic * row_vecs, base, row_vecs, lane);
 
-    const int le = floormod(e, nle, magic);
-    if (lane == 0) s_le[wave] = le;
-    lds_barrier();
+    const int R = rows_known();
     int rle[ROWS];
 #pragma unroll
-    for (int r = 0; r < ROWS; ++r) rle[r] = s_le[r];
+    for (int r = 0; r < ROWS; ++r) rle[r] = floormod(re[r], nle, magic);
     int cnt[ROWS];
-    scan.finish(key, [&](int r, int e2, int i2) {
+    scan.finish(key, min(i0 + ROWS - 1, R), [&](int r, int e2, int i2) {
       return (floormod(e2, nle, magic) == rle[r]) & (i2 < i0 + r);
     }, cnt);
-    const int pos = rows_reduce(cnt, part, wave, lane);
+    const int pos = rows_reduce(cnt, part, parity++, wave, lane);
 
-    if (valid && pos < max_recv) {
+    if (i < R && pos < max_recv) {
+      int le = 0;
+#pragma unroll
+      for (int r = 0; r < ROWS; ++r) le = r == wave ? rle[r] : le;
       const size_t row = (size_t)le * max_recv + pos;
       p.template store<(MOE_A2A_NT_RECV != 0)>(expert_x + row * row_vecs, base, row_vecs, lane);
       if (c == 0 && lane < META) expert_meta[row * META + lane] = m;
     }
+    return R;
+  };
+
+  int q = blockIdx.x - nle;
+  int R;
+  // only groups that lie wholly below the bound: their rows can be read as they are
+  const int hint_items = hint_rows / ROWS * chunks;
+  if (W <= 64 && q < hint_items) {
+    const int my_count = lane < W ? max(recv_counts[lane], 0) : 0;  // in flight with the rows
+    R = move(q, hint_rows, [&] { return wave_sum(my_count); });
+    q += movers;
+  } else {
+    R = sum_counts(recv_counts, W);
   }
+  const int items = (R + ROWS - 1) / ROWS * chunks;
+  for (; q < items; q += movers) move(q, R, [&] { return R; });
 }
 
 // ---------------------------------------------------------------- expert-major stream helpers
@@ -602,8 +634,7 @@ __global__ __launch_bounds__(64 * ROWS) void combine_send_kernel(
     const int* __restrict__ expert_num_tokens, int nle, int max_recv, int W, int row_vecs,
     int chunks, V* __restrict__ send_buf, int* __restrict__ send_meta,
     int* __restrict__ send_counts) {
-  __shared__ int part[ROWS * ROWS];
-  __shared__ int s_d[ROWS];
+  __shared__ int part[2 * ROWS * ROWS];
   __shared__ int pre[SMALL ? 1 : MAX_LOCAL_EXPERTS + 1];
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
 
@@ -619,6 +650,18 @@ __global__ __launch_bounds__(64 * ROWS) void combine_send_kernel(
   Keys key;
   if constexpr (SMALL) key = Keys{my_excl, expert_meta, nle, 32, max_recv};
   else key = Keys{pre, expert_meta, nle, top_step(nle), max_recv};
+  // padded row index of stream row g (wave-uniform g < R)
+  auto padded_row = [&](int g) -> size_t {
+    int le, first;
+    if constexpr (SMALL) {
+      le = __popcll(__ballot(my_incl <= g));
+      first = __builtin_amdgcn_readlane(my_excl, le);
+    } else {
+      le = expert_of(pre, nle, key.top, g);
+      first = pre[le];
+    }
+    return (size_t)le * max_recv + (g - first);
+  };
 
   if ((int)blockIdx.x < W) {
     const int me = blockIdx.x;
@@ -630,40 +673,29 @@ __global__ __launch_bounds__(64 * ROWS) void combine_send_kernel(
 
   const int groups = (R + ROWS - 1) / ROWS;
   const int items = groups * chunks, movers = gridDim.x - W;
-  for (int q = blockIdx.x - W; q < items; q += movers) {
+  int parity = 0;
+  for (int q = blockIdx.x - W; q < items; q += movers, ++parity) {
     const int grp = chunks == 1 ? q : q / chunks, c = q - grp * chunks;
-    const int g = grp * ROWS + wave;
+    const int g0 = grp * ROWS, g = g0 + wave;
     const bool valid = g < R;
-    const int gc = min(g, R - 1);
     const int base = c * (64 * NVW);
-    int le, first;
-    if constexpr (SMALL) {
-      le = __popcll(__ballot(my_incl <= gc));
-      first = __builtin_amdgcn_readlane(my_excl, le);
-    } else {
-      le = expert_of(pre, nle, key.top, gc);
-      first = pre[le];
-    }
-    const size_t row = (size_t)le * max_recv + (gc - first);
 
+    // origin rank of every row of the group, read by every wave (no exchange)
+    int rd[ROWS];
+#pragma unroll
+    for (int r = 0; r < ROWS; ++r) rd[r] = expert_meta[padded_row(min(g0 + r, R - 1)) * META + 1];
+    const size_t row = padded_row(min(g, R - 1));
     int m = 0;
     if (c == 0 && lane < META) m = expert_meta[row * META + lane];
-    const int d = expert_meta[row * META + 1];
     RowsScan<Keys> scan(R, key);
     WavePayload<V, NVW> p;
     p.load(expert_y + row * row_vecs, base, row_vecs, lane);
 
-    if (lane == 0) s_d[wave] = d;
-    lds_barrier();
-    int rd[ROWS];
-#pragma unroll
-    for (int r = 0; r < ROWS; ++r) rd[r] = s_d[r];
-    const int g0 = grp * ROWS;
     int cnt[ROWS];
-    scan.finish(key, [&](int r, int d2, int g2) {
+    scan.finish(key, R, [&](int r, int d2, int g2) {
       return (d2 < rd[r]) | ((d2 == rd[r]) & (g2 < g0 + r));
     }, cnt);
-    const int slot = rows_reduce(cnt, part, wave, lane);
+    const int slot = rows_reduce(cnt, part, parity, wave, lane);
 
     if (valid) {
       p.template store<(MOE_A2A_NT_CSEND != 0)>(send_buf + (size_t)slot * row_vecs, base, row_vecs, lane);
@@ -755,20 +787,61 @@ struct PairAcc {
 // The workgroup finds the rows addressed to its token by scanning the src_token
 // column of the arriving meta rows, orders them by arrival index, then walks
 // them in that order with all rows of a batch loaded up front.
+//
+// `hint_rows` rows of recv_meta are readable whatever the counts say: the first
+// batch of the scan is loaded before the true row count R is known (the counts
+// are loaded at the same time); rows at or past R are ignored.
+
+// Compare-exchange of two (row, k) pairs by row.
+__device__ __forceinline__ void order_pair(int& ra, int& ka, int& rb, int& kb) {
+  const bool swap = rb < ra;
+  const int r = swap ? rb : ra, k = swap ? kb : ka;
+  rb = swap ? ra : rb; kb = swap ? ka : kb;
+  ra = r; ka = k;
+}
+
 template <typename V, int DT, int BLK, int NV>
 __global__ __launch_bounds__(BLK) void combine_recv_kernel(
     const V* __restrict__ recv_buf, const int* __restrict__ recv_meta,
-    const int* __restrict__ recv_counts, int W, const float* __restrict__ weights, int T, int K,
-    int row_vecs, int chunks, V* __restrict__ out, int accumulate) {
+    const int* __restrict__ recv_counts, int W, int hint_rows, const float* __restrict__ weights,
+    int T, int K, int row_vecs, int chunks, V* __restrict__ out, int accumulate) {
   constexpr int N = Words<V>::N;
+  constexpr int FAST = 8;  // addends ordered in registers
   __shared__ int hit_row[COMBINE_CAP], hit_k[COMBINE_CAP];
   __shared__ int ord_row[COMBINE_CAP];
   __shared__ float ord_w[COMBINE_CAP];
   __shared__ float wts[COMBINE_WEIGHTS];
   __shared__ int nhit;
-  const int tid = threadIdx.x;
-  const int R = sum_counts(recv_counts, W);
+  const int tid = threadIdx.x, lane = tid & 63;
   const int kw = min(K, COMBINE_WEIGHTS);
+  const bool lanes_hold_counts = W <= 64;
+  const int my_count = lanes_hold_counts && lane < W ? max(recv_counts[lane], 0) : 0;
+  int R = -1;  // not known yet
+
+  // rows [lo, hi) of the arriving stream: note the ones addressed to token t
+  auto scan = [&](int t, int lo, int hi) {
+    for (int b = lo; b < hi; b += SCAN_UNROLL * BLK) {
+      int key[SCAN_UNROLL], kk[SCAN_UNROLL];
+#pragma unroll
+      for (int u = 0; u < SCAN_UNROLL; ++u) {
+        const int* m = recv_meta + (size_t)min(b + tid + u * BLK, hi - 1) * META;
+        key[u] = m[2];
+        kk[u] = m[3];
+      }
+      if (R < 0) R = lanes_hold_counts ? wave_sum(my_count) : sum_counts(recv_counts, W);
+#pragma unroll
+      for (int u = 0; u < SCAN_UNROLL; ++u) {
+        const int row = b + tid + u * BLK;
+        if (row < min(hi, R) && key[u] == t) {
+          const int p = atomicAdd(&nhit, 1);
+          if (p < COMBINE_CAP) {
+            hit_row[p] = row;
+            hit_k[p] = kk[u];
+          }
+        }
+      }
+    }
+  };
 
   const int items = T * chunks;
   for (int q = blockIdx.x; q < items; q += gridDim.x) {
@@ -791,31 +864,60 @@ __global__ __launch_bounds__(BLK) void combine_recv_kernel(
 
     if (tid == 0) nhit = 0;
     lds_barrier();
-    for (int i = tid; i < R; i += SCAN_UNROLL * BLK) {
-      int key[SCAN_UNROLL], kk[SCAN_UNROLL];
-#pragma unroll
-      for (int u = 0; u < SCAN_UNROLL; ++u) {
-        const int* m = recv_meta + (size_t)min(i + u * BLK, R - 1) * META;
-        key[u] = m[2];
-        kk[u] = m[3];
-      }
-#pragma unroll
-      for (int u = 0; u < SCAN_UNROLL; ++u) {
-        const int row = i + u * BLK;
-        if (row < R && key[u] == t) {
-          const int p = atomicAdd(&nhit, 1);
-          if (p < COMBINE_CAP) {
-            hit_row[p] = row;
-            hit_k[p] = kk[u];
-          }
-        }
-      }
+    if (R < 0) {
+      // first item: one batch below the readable bound goes out before R is known
+      const int spec = min(hint_rows, SCAN_UNROLL * BLK);
+      scan(t, 0, spec);
+      if (R < 0) R = lanes_hold_counts ? wave_sum(my_count) : sum_counts(recv_counts, W);
+      scan(t, spec, R);
+    } else {
+      scan(t, 0, R);
     }
     if (tid < kw) wts[tid] = wreg;
     lds_barrier();
     const int n = nhit;
 
-    if (n <= COMBINE_CAP) {
+    if (n <= FAST) {
+      // order the (at most 8) hits by arrival index in registers, every lane for itself
+      int hr[FAST], hk[FAST];
+#pragma unroll
+      for (int u = 0; u < FAST; ++u) {
+        hr[u] = u < n ? hit_row[u] : INT_MAX;
+        hk[u] = u < n ? hit_k[u] : -1;
+      }
+#define MOE_A2A_CE(a, b) order_pair(hr[a], hk[a], hr[b], hk[b])
+      MOE_A2A_CE(0, 1); MOE_A2A_CE(2, 3); MOE_A2A_CE(4, 5); MOE_A2A_CE(6, 7);
+      MOE_A2A_CE(0, 2); MOE_A2A_CE(1, 3); MOE_A2A_CE(4, 6); MOE_A2A_CE(5, 7);
+      MOE_A2A_CE(1, 2); MOE_A2A_CE(5, 6);
+      MOE_A2A_CE(0, 4); MOE_A2A_CE(1, 5); MOE_A2A_CE(2, 6); MOE_A2A_CE(3, 7);
+      MOE_A2A_CE(2, 4); MOE_A2A_CE(3, 5);
+      MOE_A2A_CE(1, 2); MOE_A2A_CE(3, 4); MOE_A2A_CE(5, 6);
+#undef MOE_A2A_CE
+      if (n > 0) {
+        V v[FAST][NV];
+        float w[FAST];
+#pragma unroll
+        for (int u = 0; u < FAST; ++u) {
+          const int k = hk[u];
+          const bool ok = (u < n) & (k >= 0) & (k < K);
+          if (!ok) hr[u] = -1;
+          w[u] = !ok ? 0.0f : k < kw ? wts[k] : weights[(size_t)t * K + k];
+          const int row = ok ? hr[u] : 0;  // row 0 exists: n > 0; loaded and not used
+#pragma unroll
+          for (int j = 0; j < NV; ++j)
+            v[u][j] = recv_buf[(size_t)row * row_vecs + min(base + j * BLK + tid, row_vecs - 1)];
+        }
+#pragma unroll
+        for (int u = 0; u < FAST; ++u) {
+          if (hr[u] >= 0) {
+#pragma unroll
+            for (int j = 0; j < NV; ++j)
+#pragma unroll
+              for (int e = 0; e < N; ++e) acc[j][e].step(get_word(v[u][j], e), w[u]);
+          }
+        }
+      }
+    } else if (n <= COMBINE_CAP) {
       if (tid < n) {  // order the hits by arrival index
         const int me = hit_row[tid];
         int r = 0;
@@ -1094,8 +1196,8 @@ int moe_a2a_dispatch_recv(const moe_a2a_shape* s, const void* recv_buf, const in
   hipStream_t st = (hipStream_t)stream;
 #define LAUNCH(V, NVW)                                                                      \
   dispatch_recv_kernel<V, NVW><<<grid, 64 * ROWS, 0, st>>>(                                 \
-      (const V*)recv_buf, recv_meta, recv_counts, s->world_size, g.nle, g.magic, g.max_recv, \
-      g.row_vecs, g.wchunks, expert_num_tokens, (V*)expert_x, expert_meta)
+      (const V*)recv_buf, recv_meta, recv_counts, s->world_size, rows_hint, g.nle, g.magic,  \
+      g.max_recv, g.row_vecs, g.wchunks, expert_num_tokens, (V*)expert_x, expert_meta)
   MOE_A2A_FOR_WAVE_KERNEL(g, LAUNCH);
 #undef LAUNCH
   return launch_status();
@@ -1130,40 +1232,33 @@ int moe_a2a_combine_send(const moe_a2a_shape* s, const void* expert_y, const int
 }
 
 int moe_a2a_combine_recv(const moe_a2a_shape* s, const void* recv_buf, const int32_t* recv_meta,
-                         const int32_t* recv_counts, const float* weights, int32_t num_tokens,
-                         void* out_tokens, int32_t accumulate, int32_t dtype, void* stream) {
-  if (!shape_ok(s) || num_tokens < 0 || num_tokens > s->max_num_tokens || !recv_counts)
+                         const int32_t* recv_counts, int32_t rows_hint, const float* weights,
+                         int32_t num_tokens, void* out_tokens, int32_t accumulate, int32_t dtype,
+                         void* stream) {
+  if (!shape_ok(s) || num_tokens < 0 || num_tokens > s->max_num_tokens || !recv_counts ||
+      rows_hint < 0)
     return MOE_A2A_EINVAL;
   if (dtype != MOE_A2A_F16 && dtype != MOE_A2A_BF16) return MOE_A2A_EINVAL;
   if (num_tokens == 0) return MOE_A2A_OK;
   if (!recv_buf || !recv_meta || !weights || !out_tokens) return MOE_A2A_EINVAL;
   if (!all_aligned(2, recv_buf, out_tokens)) return MOE_A2A_EALIGN;
   const Geometry g = geometry(s, recv_buf, out_tokens);
-  // wide rows: one 1024-lane workgroup per token scans the arrivals once; narrower rows use
-  // 256 lanes with one or two vector columns each
-#ifndef MOE_A2A_COMBINE_WIDE
-#define MOE_A2A_COMBINE_WIDE 256
-#endif
-#ifndef MOE_A2A_COMBINE_NV
-#define MOE_A2A_COMBINE_NV 1
-#endif
-  const int blk = g.row_vecs >= 768 ? MOE_A2A_COMBINE_WIDE : BLOCK;
-  const int nv = g.row_vecs >= 768 ? MOE_A2A_COMBINE_NV : g.row_vecs <= BLOCK ? 1 : 2;
-  const int chunks = (g.row_vecs + blk * nv - 1) / (blk * nv);
+  // 256 lanes per (token, chunk), one vector column each; rows of at most 512
+  // vectors are not split, their lanes take two columns
+  const int nv = g.row_vecs > BLOCK && g.row_vecs <= 2 * BLOCK ? 2 : 1;
+  const int chunks = (g.row_vecs + BLOCK * nv - 1) / (BLOCK * nv);
   if (!items_fit(num_tokens, chunks)) return MOE_A2A_EINVAL;
   const int grid = mover_blocks((long long)num_tokens * chunks);
   hipStream_t st = (hipStream_t)stream;
   const int K = s->experts_per_token, W = s->world_size;
 #define LAUNCH(V, DT, BLK, NV)                                                               \
   combine_recv_kernel<V, DT, BLK, NV><<<grid, BLK, 0, st>>>(                                 \
-      (const V*)recv_buf, recv_meta, recv_counts, W, weights, num_tokens, K, g.row_vecs,     \
-      chunks, (V*)out_tokens, accumulate)
-#define PICK_SHAPE(V, DT)                                  \
-  do {                                                     \
-    if (blk == 1024) { LAUNCH(V, DT, 1024, 1); }           \
-    else if (blk == 512) { LAUNCH(V, DT, 512, 1); }        \
-    else if (nv == 1) { LAUNCH(V, DT, BLOCK, 1); }         \
-    else { LAUNCH(V, DT, BLOCK, 2); }                      \
+      (const V*)recv_buf, recv_meta, recv_counts, W, rows_hint, weights, num_tokens, K,      \
+      g.row_vecs, chunks, (V*)out_tokens, accumulate)
+#define PICK_SHAPE(V, DT)                       \
+  do {                                          \
+    if (nv == 1) { LAUNCH(V, DT, BLOCK, 1); }   \
+    else { LAUNCH(V, DT, BLOCK, 2); }           \
   } while (0)
   if (g.vec16) {
     if (dtype == MOE_A2A_BF16) PICK_SHAPE(b128, MOE_A2A_BF16);

@@ -14,10 +14,13 @@
  *   - nothing is allocated, freed or cleared by the library; every output
  *     buffer is owned by the caller; no entry point synchronises the host;
  *   - `stream` is a hipStream_t passed as void*; NULL is the null stream;
- *   - every `rows_hint` is a host-side upper-bound guess of the number of
- *     rows the call will move. It only sizes the launch: kernels read the
- *     true row count from device memory and stride over it, so a wrong hint
- *     costs time, never correctness;
+ *   - every `rows_hint` is a host-side guess of the number of rows the call
+ *     will move. Kernels read the true row count from device memory and
+ *     stride over it, so a hint that is too small or too large costs time,
+ *     never correctness. One rule comes with it: the input row and meta
+ *     buffers of the call must be readable for `rows_hint` rows (pass at most
+ *     the capacity they were allocated with). Rows between the true count and
+ *     the hint may be read before the count is known; they are never used;
  *   - return value: MOE_A2A_OK (0) or a negative MOE_A2A_E* code. Argument
  *     errors are detected before anything is launched.
  *
@@ -146,9 +149,9 @@ int moe_a2a_combine_send(const moe_a2a_shape* shape, const void* expert_y,
  */
 int moe_a2a_combine_recv(const moe_a2a_shape* shape, const void* recv_buf,
                          const int32_t* recv_meta, const int32_t* recv_counts,
-                         const float* weights, int32_t num_tokens,
-                         void* out_tokens, int32_t accumulate, int32_t dtype,
-                         void* stream);
+                         int32_t rows_hint, const float* weights,
+                         int32_t num_tokens, void* out_tokens,
+                         int32_t accumulate, int32_t dtype, void* stream);
 
 /*
  * Stand-in for the expert computation between dispatch and combine.
