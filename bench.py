@@ -38,6 +38,14 @@ if str(ROOT) not in sys.path:
 HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published
 META_BYTES = 20
 
+# HBM bytes per launch of rank 0's kernels on workload C4 (seed 2025), from rocprofv3 FETCH_SIZE and
+# WRITE_SIZE scaled by what the same counters read for the exchange copy of known size
+# (profiles/c4_rank0_hbm_traffic.md). Other workloads have no committed counter run: traffic is null.
+MEASURED_TRAFFIC_BYTES = {
+    ("C4", 2025): {"dispatch_send": 33.14e6, "dispatch_recv": 57.79e6,
+                   "combine_send": 57.78e6, "combine_recv": 33.02e6},
+}
+
 
 def parse_args():
     ap = argparse.ArgumentParser()
@@ -246,7 +254,8 @@ def main():
         "roofline": {
             "bound": "hbm", "kernel": dominant,
             "achieved": kern[dominant]["gbps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-            "frac": kern[dominant]["frac"], "traffic": None,
+            "frac": kern[dominant]["frac"],
+            "traffic": MEASURED_TRAFFIC_BYTES.get((args.workload, args.seed), {}).get(dominant),
         },
         "result_identical_to_setup_run": same_as_setup,
     }
