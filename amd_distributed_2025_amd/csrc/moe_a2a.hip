@@ -826,7 +826,7 @@ __global__ __launch_bounds__(BLK) void combine_recv_kernel(
       for (int u = 0; u < SCAN_UNROLL; ++u) {
         const int* m = recv_meta + (size_t)min(b + tid + u * BLK, hi - 1) * META;
         key[u] = m[2];
-        kk[u] = m[3];
+        kk[u] = m[3];  // same cache line; a dependent load for the hits alone costs more
       }
       if (R < 0) R = lanes_hold_counts ? wave_sum(my_count) : sum_counts(recv_counts, W);
 #pragma unroll
@@ -1245,7 +1245,10 @@ int moe_a2a_combine_recv(const moe_a2a_shape* s, const void* recv_buf, const int
   const Geometry g = geometry(s, recv_buf, out_tokens);
   // 256 lanes per (token, chunk), one vector column each; rows of at most 512
   // vectors are not split, their lanes take two columns
-  const int nv = g.row_vecs > BLOCK && g.row_vecs <= 2 * BLOCK ? 2 : 1;
+  // 256 lanes per (token, chunk) with one vector column each for rows up to 256 vectors and two
+  // columns beyond. Every workgroup of a token repeats the scan of the arrivals, so fewer, fatter
+  // chunks win until the registers of a lane (8 addends x columns in flight) run out.
+  const int nv = g.row_vecs > BLOCK ? 2 : 1;
   const int chunks = (g.row_vecs + BLOCK * nv - 1) / (BLOCK * nv);
   if (!items_fit(num_tokens, chunks)) return MOE_A2A_EINVAL;
   const int grid = mover_blocks((long long)num_tokens * chunks);
