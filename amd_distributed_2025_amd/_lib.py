@@ -39,6 +39,7 @@ _SP = C.POINTER(Shape)
 # name -> argument types; every function returns int (status) unless noted
 SIGNATURES = {
     "moe_a2a_dispatch_send": [_SP, _P, _P, _I, _P, _P, _P, _P, _P],
+    "moe_a2a_plan_send": [_SP, _P, _I, _P, _P, _P, _P, _P, _P],
     "moe_a2a_dispatch_recv": [_SP, _P, _P, _P, _I, _P, _P, _P, _P],
     "moe_a2a_combine_send": [_SP, _P, _P, _P, _I, _P, _P, _P, _P],
     "moe_a2a_combine_recv": [_SP, _P, _P, _P, _I, _P, _I, _P, _I, _I, _P],

@@ -116,6 +116,24 @@ class HIPAllToAll:
         out = (counts, buf[:S], meta[:S])
         return out + (slots[:S],) if want_slots else out
 
+    def plan_send(self, indices: torch.Tensor):
+        """Counts, offsets and index maps of the send order, without moving rows.
+        Returns (rank_counts[W], rank_offsets[W+1], expert_counts[E], dst_slot[T*K], src_entry[T*K])."""
+        cfg = self.cfg
+        T, K = indices.shape
+        if K != cfg.experts_per_token:
+            raise ValueError("plan_send: indices do not match the config")
+        _need(indices, torch.int32, self.device, "indices")
+        S = T * K
+        rc = self._buf("plan_rank_counts", (self.world_size,), torch.int32)
+        ro = self._buf("plan_rank_offsets", (self.world_size + 1,), torch.int32)
+        ec = self._buf("plan_expert_counts", (cfg.num_experts,), torch.int32)
+        ds = self._buf("plan_dst_slot", (self.max_rows_out,), torch.int32)
+        se = self._buf("plan_src_entry", (self.max_rows_out,), torch.int32)
+        _lib.call("moe_a2a_plan_send", self._shape_ref, _ptr(indices), T, _ptr(rc), _ptr(ro), _ptr(ec),
+                  _ptr(ds), _ptr(se), _stream(self.device))
+        return rc, ro, ec, ds[:S], se[:S]
+
     def dispatch_recv(self, recv_counts, recv_buf, recv_meta, rows_hint: Optional[int] = None):
         """Received stream -> (expert_num_tokens[nle], expert_x[nle,max_recv,H],
         expert_meta[nle,max_recv,5]); rows past expert_num_tokens[le] are not written."""

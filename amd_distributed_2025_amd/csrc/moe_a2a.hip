@@ -402,6 +402,122 @@ __global__ __launch_bounds__(64 * ROWS) void dispatch_send_kernel(
   }
 }
 
+// ---------------------------------------------------------------- send plan (counts, offsets, maps)
+//
+// The stable counting sort of stage 1 made explicit, for callers that want the
+// plan without moving rows (a sender that writes into a peer's buffer, a
+// debugger): rows per destination rank and per expert, the exclusive offsets
+// of the destinations, and both index maps. One workgroup of 16 waves walks
+// the (t, k) stream in tiles of 1024 entries:
+//   pass 1  per-wave privatised LDS histograms of the destinations (no two
+//           waves touch the same counters), one shared LDS histogram of the
+//           expert ids; a wave64 exclusive scan turns the destination totals
+//           into offsets;
+//   pass 2  inside a wave, an entry's rank among the earlier lanes with the
+//           same destination comes from a ballot per destination present in
+//           the wave; the waves of a tile are ordered by a prefix over their
+//           per-destination counts, tiles by a running base per destination.
+// slot(i) = offset[d] + #earlier entries with destination d — the order of
+// all2all/reference.py:79-86,93.
+
+constexpr int PLAN_BLOCK = 1024;
+constexpr int PLAN_WAVES = PLAN_BLOCK / 64;
+constexpr int PLAN_MAX_RANKS = 64;      // destinations kept per wave in LDS
+constexpr int PLAN_MAX_EXPERTS = 8192;  // shared expert histogram in LDS
+
+__global__ __launch_bounds__(PLAN_BLOCK) void plan_send_kernel(
+    const int* __restrict__ indices, int S, int nle, int E, int W, uint32_t magic,
+    int* __restrict__ rank_counts, int* __restrict__ rank_offsets, int* __restrict__ expert_counts,
+    int* __restrict__ dst_slot, int* __restrict__ src_entry) {
+  __shared__ int wave_hist[PLAN_WAVES][PLAN_MAX_RANKS];
+  __shared__ int base[PLAN_MAX_RANKS];        // next free slot of each destination
+  __shared__ int expert_hist[PLAN_MAX_EXPERTS];
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const unsigned long long lanes_below = lane == 0 ? 0ull : (~0ull >> (64 - lane));
+
+  auto dest_of = [&](int e) { return nle == 1 ? e : (int)__umulhi((uint32_t)e, magic); };
+  auto in_range = [&](int e) { return (e >= 0) & (e < E); };
+
+  // ---- pass 1: histograms
+  for (int i = tid; i < PLAN_WAVES * PLAN_MAX_RANKS; i += PLAN_BLOCK) (&wave_hist[0][0])[i] = 0;
+  for (int i = tid; i < E; i += PLAN_BLOCK) expert_hist[i] = 0;
+  lds_barrier();
+  for (int b = 0; b < S; b += PLAN_BLOCK) {
+    const int i = b + tid;
+    const int e = i < S ? indices[i] : -1;
+    if (in_range(e)) {
+      atomicAdd(&expert_hist[e], 1);
+      // lanes of one wave that share a destination add their count once
+      const int d = dest_of(e);
+      unsigned long long todo = __ballot(1);
+      while (todo) {
+        const int leader = __builtin_amdgcn_readfirstlane(d);
+        const unsigned long long same = __ballot(d == leader);
+        if (d == leader) {
+          if ((same & lanes_below) == 0) wave_hist[wave][leader] += __popcll(same);
+          break;
+        }
+        todo &= ~same;
+      }
+    }
+  }
+  lds_barrier();
+  for (int i = tid; i < E; i += PLAN_BLOCK) expert_counts[i] = expert_hist[i];
+  if (wave == 0) {  // destination totals -> exclusive offsets with a wave64 scan
+    int total = 0;
+    if (lane < W) {
+#pragma unroll
+      for (int w = 0; w < PLAN_WAVES; ++w) total += wave_hist[w][lane];
+    }
+    const int incl = wave_inclusive_scan(total);
+    if (lane < W) {
+      rank_counts[lane] = total;
+      rank_offsets[lane] = incl - total;
+      base[lane] = incl - total;
+    }
+    if (lane == W - 1 || (W == 64 && lane == 63)) rank_offsets[W] = incl;
+  }
+  lds_barrier();
+
+  // ---- pass 2: stable slots, tile by tile
+  for (int b = 0; b < S; b += PLAN_BLOCK) {
+    for (int i = tid; i < PLAN_WAVES * PLAN_MAX_RANKS; i += PLAN_BLOCK) (&wave_hist[0][0])[i] = 0;
+    lds_barrier();
+    const int i = b + tid;
+    const int e = i < S ? indices[i] : -1;
+    const bool ok = in_range(e);
+    const int d = ok ? dest_of(e) : -1;
+    int rank_in_wave = 0;
+    unsigned long long todo = __ballot(ok);
+    while (todo) {  // every lane of the wave runs the same number of rounds
+      const int first = __ffsll((long long)todo) - 1;
+      const int leader = __builtin_amdgcn_readlane(d, first);
+      const unsigned long long same = __ballot(ok && d == leader);
+      if (ok && d == leader) {
+        rank_in_wave = __popcll(same & lanes_below);
+        if (rank_in_wave == 0) wave_hist[wave][leader] = __popcll(same);
+      }
+      todo &= ~same;
+    }
+    lds_barrier();
+    if (ok) {
+      int before = base[d];
+      for (int w = 0; w < wave; ++w) before += wave_hist[w][d];
+      const int slot = before + rank_in_wave;
+      dst_slot[i] = slot;
+      src_entry[slot] = i;
+    }
+    lds_barrier();
+    if (tid < W) {
+      int t = 0;
+#pragma unroll
+      for (int w = 0; w < PLAN_WAVES; ++w) t += wave_hist[w][tid];
+      base[tid] += t;
+    }
+    lds_barrier();
+  }
+}
+
 // ---------------------------------------------------------------- stage 2: dispatch, receive side
 //
 // grid = nle counting workgroups (rows per local expert) followed by one
@@ -1177,6 +1293,23 @@ int moe_a2a_dispatch_send(const moe_a2a_shape* s, const void* x, const int32_t* 
       g.magic, s->rank, g.row_vecs, g.wchunks, (V*)send_buf, send_meta, send_counts, send_slot)
   MOE_A2A_FOR_WAVE_KERNEL(g, LAUNCH);
 #undef LAUNCH
+  return launch_status();
+}
+
+int moe_a2a_plan_send(const moe_a2a_shape* s, const int32_t* indices, int32_t num_tokens,
+                      int32_t* rank_counts, int32_t* rank_offsets, int32_t* expert_counts,
+                      int32_t* dst_slot, int32_t* src_entry, void* stream) {
+  if (!shape_ok(s) || num_tokens < 0 || num_tokens > s->max_num_tokens || !rank_counts ||
+      !rank_offsets || !expert_counts)
+    return MOE_A2A_EINVAL;
+  if (s->world_size > PLAN_MAX_RANKS || s->num_experts > PLAN_MAX_EXPERTS) return MOE_A2A_EINVAL;
+  const long long S = (long long)num_tokens * s->experts_per_token;
+  if (S > INT_MAX / 2) return MOE_A2A_EINVAL;
+  if (S > 0 && (!indices || !dst_slot || !src_entry)) return MOE_A2A_EINVAL;
+  const Geometry g = geometry(s);
+  plan_send_kernel<<<1, PLAN_BLOCK, 0, (hipStream_t)stream>>>(
+      indices, (int)S, g.nle, s->num_experts, s->world_size, g.magic, rank_counts, rank_offsets,
+      expert_counts, dst_slot, src_entry);
   return launch_status();
 }
 

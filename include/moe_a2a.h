@@ -90,6 +90,26 @@ int moe_a2a_dispatch_send(const moe_a2a_shape* shape, const void* x,
                           void* stream);
 
 /*
+ * The plan of the send side without moving any row: counts, offsets and both
+ * index maps of the stable sort that moe_a2a_dispatch_send applies
+ * (all2all/reference.py:79-86,93: entries grouped by destination rank, inside
+ * a group in (t, k) order).
+ *
+ *   indices       [num_tokens, K] int32
+ *   rank_counts   [W]   out: entries per destination rank (= send_counts)
+ *   rank_offsets  [W+1] out: exclusive prefix of rank_counts; [W] = total
+ *   expert_counts [E]   out: entries per global expert id
+ *   dst_slot      [num_tokens*K] out: send row of entry t*K+k
+ *   src_entry     [num_tokens*K] out: entry t*K+k held by each send row
+ * Entries whose expert id is outside [0, E) are left out of every output.
+ * Limits: W <= 64, E <= 8192 (MOE_A2A_EINVAL beyond).
+ */
+int moe_a2a_plan_send(const moe_a2a_shape* shape, const int32_t* indices,
+                      int32_t num_tokens, int32_t* rank_counts,
+                      int32_t* rank_offsets, int32_t* expert_counts,
+                      int32_t* dst_slot, int32_t* src_entry, void* stream);
+
+/*
  * Dispatch, receive side: received stream -> expert-major buffers.
  * Replaces all2all/reference.py:123-146 (per received row:
  * le = meta[0] % nle; expert_x[le, cnt[le]++] = row).

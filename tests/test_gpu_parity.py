@@ -344,3 +344,43 @@ def test_graph_replays_match_eager():
         graph.replay()
         torch.cuda.synchronize()
         assert torch.equal(y[: d0.num_tokens], eager[0]), f"replay {i}"
+
+
+@pytest.mark.parametrize("name", ["C1", "C2", "C3", "C4", "C5"])
+def test_send_plan_counts_offsets_and_maps(name):
+    """The explicit plan (per-rank and per-expert counts, offsets, dst and src maps)
+    equals the oracle's stable order, and the fused dispatch_send uses the same slots."""
+    print(f"plan {name}", flush=True)
+    world = generate_world(WORKLOADS[name], 606)
+    cfg = world[0][0]
+    W = len(world)
+    nle = cfg.num_experts // W
+    lw = LocalWorld(cfg, W, device=DEV)
+    for r in (0, W - 1):
+        d = world[r][1].to(DEV)
+        rc, ro, ec, dst, src = lw.ranks[r].plan_send(d.indices)
+        _, _, _, slots = lw.ranks[r].dispatch_send(d.x, d.indices, want_slots=True)
+        torch.cuda.synchronize()
+        counts, order = orc.send_order(d.indices.cpu().numpy(), nle, W)
+        S = order.size
+        inv = np.empty(S, np.int64); inv[order] = np.arange(S)
+        assert np.array_equal(rc.cpu().numpy(), counts)
+        assert np.array_equal(ro.cpu().numpy(), np.concatenate([[0], np.cumsum(counts)]))
+        assert np.array_equal(ec.cpu().numpy(), np.bincount(d.indices.cpu().numpy().ravel(), minlength=cfg.num_experts))
+        assert np.array_equal(src.cpu().numpy(), order)
+        assert np.array_equal(dst.cpu().numpy(), inv)
+        assert np.array_equal(slots.cpu().numpy(), inv)
+
+
+def test_send_plan_many_tiles_and_ragged_tail():
+    """More entries than one 1024-entry tile, a tail that does not fill a wave, 64 ranks."""
+    cfg = MoEConfig(128, 7, 16, 333, torch.bfloat16, torch.bfloat16)
+    a = LocalWorld(cfg, 64, device=DEV).ranks[5]
+    rng = np.random.default_rng(8)
+    idx = np.stack([rng.permutation(128)[:7] for _ in range(333)]).astype(np.int32)
+    rc, ro, ec, dst, src = a.plan_send(torch.from_numpy(idx).to(DEV))
+    torch.cuda.synchronize()
+    counts, order = orc.send_order(idx, 2, 64)
+    assert np.array_equal(rc.cpu().numpy(), counts)
+    assert np.array_equal(src.cpu().numpy(), order)
+    assert np.array_equal(ro.cpu().numpy()[-1:], [333 * 7])
