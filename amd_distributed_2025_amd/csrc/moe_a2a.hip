@@ -940,9 +940,12 @@ __global__ __launch_bounds__(BLK) void combine_recv_kernel(
       int key[SCAN_UNROLL], kk[SCAN_UNROLL];
 #pragma unroll
       for (int u = 0; u < SCAN_UNROLL; ++u) {
-        const int* m = recv_meta + (size_t)min(b + tid + u * BLK, hi - 1) * META;
-        key[u] = m[2];
-        kk[u] = m[3];  // same cache line; a dependent load for the hits alone costs more
+        // src_token and src_k with one 8-byte load (4-byte aligned, which global loads accept);
+        // fetching src_k for the hits alone with a dependent load costs more than it saves
+        int tk[2];
+        __builtin_memcpy(tk, recv_meta + (size_t)min(b + tid + u * BLK, hi - 1) * META + 2, 8);
+        key[u] = tk[0];
+        kk[u] = tk[1];
       }
       if (R < 0) R = lanes_hold_counts ? wave_sum(my_count) : sum_counts(recv_counts, W);
 #pragma unroll

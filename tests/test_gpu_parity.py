@@ -384,3 +384,24 @@ def test_send_plan_many_tiles_and_ragged_tail():
     assert np.array_equal(rc.cpu().numpy(), counts)
     assert np.array_equal(src.cpu().numpy(), order)
     assert np.array_equal(ro.cpu().numpy()[-1:], [333 * 7])
+
+
+def test_random_small_jobs():
+    """A seeded sweep over small job shapes (world sizes 1..16, few to many local
+    experts, row lengths on and off the 16-byte path, fp16 and bf16, all routing
+    and token-count rules): every intermediate of every rank against the oracle."""
+    rng = np.random.default_rng(20251125)
+    for case in range(40):
+        W = int(rng.choice([1, 2, 3, 4, 8, 16]))
+        nle = int(rng.choice([1, 2, 5, 32, 65, 130]))
+        E = W * nle
+        K = int(rng.integers(1, min(E, 9) + 1))
+        H = int(rng.choice([8, 24, 100, 256, 520, 1032, 4104]))
+        max_T = int(rng.integers(1, 40))
+        spec = dict(world_size=W, num_experts=E, experts_per_token=K, hidden_dim=H, max_num_tokens=max_T,
+                    num_tokens=str(rng.choice(["uniform", "full", "reference"])),
+                    routing=str(rng.choice(["uniform", "zipf"])),
+                    weights=str(rng.choice(["rand", "softmax"])),
+                    dtype=str(rng.choice(["bf16", "fp16"])))
+        print(f"random job {case}: {spec}", flush=True)
+        run_and_compare(generate_world(spec, 9000 + case), exact_hints=bool(case % 2))
