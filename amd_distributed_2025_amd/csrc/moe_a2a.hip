@@ -1384,7 +1384,10 @@ int moe_a2a_combine_recv(const moe_a2a_shape* s, const void* recv_buf, const int
   // 256 lanes per (token, chunk) with one vector column each for rows up to 256 vectors and two
   // columns beyond. Every workgroup of a token repeats the scan of the arrivals, so fewer, fatter
   // chunks win until the registers of a lane (8 addends x columns in flight) run out.
-  const int nv = g.row_vecs > BLOCK ? 2 : 1;
+#ifndef MOE_A2A_COMBINE_NV_WIDE
+#define MOE_A2A_COMBINE_NV_WIDE 1
+#endif
+  const int nv = g.row_vecs > 2 * BLOCK ? MOE_A2A_COMBINE_NV_WIDE : g.row_vecs > BLOCK ? 2 : 1;
   const int chunks = (g.row_vecs + BLOCK * nv - 1) / (BLOCK * nv);
   if (!items_fit(num_tokens, chunks)) return MOE_A2A_EINVAL;
   const int grid = mover_blocks((long long)num_tokens * chunks);

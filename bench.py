@@ -3,7 +3,7 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload C4] [--mode graph|eager]
 
-A step is one pass of rank 0's share of the job, everything on the device and
+A step is one pass of one rank's share of the job (rank 0 unless --rank says otherwise), everything on the device and
 on one stream:
 
     dispatch_send -> [exchange leg 0->0] -> dispatch_recv -> [expert stand-in]
@@ -42,7 +42,7 @@ META_BYTES = 20
 # WRITE_SIZE scaled by what the same counters read for the exchange copy of known size
 # (profiles/c4_rank0_hbm_traffic.md). Other workloads have no committed counter run: traffic is null.
 MEASURED_TRAFFIC_BYTES = {
-    ("C4", 2025): {"dispatch_send": 33.14e6, "dispatch_recv": 57.79e6,
+    ("C4", 2025, 0): {"dispatch_send": 33.14e6, "dispatch_recv": 57.79e6,
                    "combine_send": 57.78e6, "combine_recv": 33.02e6},
 }
 
@@ -54,6 +54,7 @@ def parse_args():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default="C4", choices=["C1", "C2", "C3", "C4", "C5"])
     ap.add_argument("--seed", type=int, default=2025)
+    ap.add_argument("--rank", type=int, default=0, help="rank whose share of the job is timed")
     ap.add_argument("--mode", default="graph", choices=["graph", "eager"],
                     help="replay a captured HIP graph of the step (default) or launch eagerly")
     ap.add_argument("--kernel-reps", type=int, default=20,
@@ -106,11 +107,15 @@ def main():
     lw = LocalWorld(cfg, W, device=dev)
     ys0 = [y.clone() for y in lw.run(data)]
     torch.cuda.synchronize()
-    a, d0, g = lw.ranks[0], data[0], lw.trace[0]
+    r0 = args.rank
+    if not 0 <= r0 < W:
+        print(f"--rank must be in [0, {W})", file=sys.stderr)
+        sys.exit(2)
+    a, d0, g = lw.ranks[r0], data[r0], lw.trace[r0]
     T = d0.num_tokens
     R = int(g["recv_counts"].sum().item())
-    own_out = int(g["send_counts"][0].item())   # rows rank 0 sends to itself
-    own_back = int(g["back_counts"][0].item())
+    own_out = int(g["send_counts"][r0].item())   # rows the rank sends to itself
+    own_back = int(g["back_counts"][r0].item())
     y = a._buf("y", (cfg.max_num_tokens, H), cfg.out_dtype)
 
     def k_dispatch_send():
@@ -172,7 +177,7 @@ def main():
     wall = time.perf_counter() - t0
     ms_per_step = wall * 1e3 / args.steps
     y_after = y[:T].clone()
-    same_as_setup = bool(torch.equal(y_after, ys0[0]))
+    same_as_setup = bool(torch.equal(y_after, ys0[r0]))
 
     # ---- per-kernel timing, in the pipeline: HIP events on the launch stream around a graph of
     # `reps` whole steps, with and without the kernel. The difference is what the kernel costs where
@@ -239,7 +244,7 @@ def main():
         "dtype": "bf16" if cfg.in_dtype == torch.bfloat16 else "f16",
         "data": "synthetic",
         "config": {
-            "workload": f"{args.workload}: rank 0 of world_size={W}, num_experts={cfg.num_experts}, "
+            "workload": f"{args.workload}: rank {r0} of world_size={W}, num_experts={cfg.num_experts}, "
                         f"experts_per_token={K}, hidden_dim={H}, num_tokens={T}, routing={wl['routing']}, "
                         f"weights={wl['weights']}, seed={args.seed}",
             "rows_sent": T * K, "rows_received": R, "mode": args.mode,
@@ -255,7 +260,7 @@ def main():
             "bound": "hbm", "kernel": dominant,
             "achieved": kern[dominant]["gbps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
             "frac": kern[dominant]["frac"],
-            "traffic": MEASURED_TRAFFIC_BYTES.get((args.workload, args.seed), {}).get(dominant),
+            "traffic": MEASURED_TRAFFIC_BYTES.get((args.workload, args.seed, r0), {}).get(dominant),
         },
         "result_identical_to_setup_run": same_as_setup,
     }
@@ -271,9 +276,9 @@ def main():
 
         def cpu_step():
             t = [time.perf_counter()]
-            rw.send_side(x_c, idx_c, 0, W, nle); t.append(time.perf_counter())
+            rw.send_side(x_c, idx_c, r0, W, nle); t.append(time.perf_counter())
             n_per, ex, em = rw.place_rows(recv_b, recv_m, nle, max_recv); t.append(time.perf_counter())
-            ey = rw.simulated_expert(ex, 0, cfg.out_dtype); t.append(time.perf_counter())
+            ey = rw.simulated_expert(ex, r0, cfg.out_dtype); t.append(time.perf_counter())
             rw.return_side(ey, em, n_per, W); t.append(time.perf_counter())
             yc = torch.zeros(cfg.max_num_tokens, H, dtype=cfg.out_dtype)
             rw.accumulate(yc, w_c, ret_b, ret_m); t.append(time.perf_counter())
@@ -289,7 +294,7 @@ def main():
         out["cpu_baseline"] = {
             "value": round(sum(med) * 1e6, 1), "unit": "us", "cores": torch.get_num_threads(),
             "kind": "port",
-            "sample": f"{len(runs)} full steps of rank 0's share of {args.workload} "
+            "sample": f"{len(runs)} full steps of rank {r0}'s share of {args.workload} "
                       f"({spent:.1f} s of CPU), median per phase",
             "hot_path_us": round(cpu_path_us, 1),
             "expert_standin_us": round(med[2] * 1e6, 1),
