@@ -141,13 +141,14 @@ class HIPAllToAll:
         _need(recv_counts, torch.int32, self.device, "recv_counts")
         _need(recv_buf, cfg.in_dtype, self.device, "recv_buf")
         _need(recv_meta, torch.int32, self.device, "recv_meta")
-        hint = min(recv_buf.shape[0], recv_meta.shape[0], self.max_rows_in if rows_hint is None else rows_hint)
+        capacity = min(recv_buf.shape[0], recv_meta.shape[0])
+        hint = min(capacity, self.max_rows_in if rows_hint is None else int(rows_hint))
         nle = self.num_local_experts
         num = self._buf("expert_num_tokens", (nle,), torch.int32)
         ex = self._buf("expert_x", (nle, self.max_recv, cfg.hidden_dim), cfg.in_dtype)
         em = self._buf("expert_meta", (nle, self.max_recv, META_DIM), torch.int32)
         _lib.call("moe_a2a_dispatch_recv", self._shape_ref, _ptr(recv_buf), _ptr(recv_meta),
-                  _ptr(recv_counts), hint, _ptr(num), _ptr(ex), _ptr(em), _stream(self.device))
+                  _ptr(recv_counts), hint, capacity, _ptr(num), _ptr(ex), _ptr(em), _stream(self.device))
         self._rows_in_hint = hint
         return num, ex, em
 
@@ -178,8 +179,8 @@ class HIPAllToAll:
         buf = self._buf("back_buf", (self.max_rows_in, cfg.hidden_dim), cfg.out_dtype)
         meta = self._buf("back_meta", (self.max_rows_in, META_DIM), torch.int32)
         _lib.call("moe_a2a_combine_send", self._shape_ref, _ptr(expert_y), _ptr(expert_meta),
-                  _ptr(expert_num_tokens), hint, _ptr(buf), _ptr(meta), _ptr(counts),
-                  _stream(self.device))
+                  _ptr(expert_num_tokens), min(hint, self.max_rows_in), self.max_rows_in, _ptr(buf),
+                  _ptr(meta), _ptr(counts), _stream(self.device))
         return counts, buf, meta
 
     def combine_recv(self, out_tokens, weights, ret_counts, ret_buf, ret_meta, accumulate: bool = True):
@@ -195,9 +196,10 @@ class HIPAllToAll:
         T = weights.shape[0]
         if out_tokens.shape[0] < T or out_tokens.shape[1] != cfg.hidden_dim:
             raise ValueError("combine: out_tokens must hold num_tokens rows of hidden_dim")
-        hint = min(ret_buf.shape[0], ret_meta.shape[0], T * cfg.experts_per_token)
+        capacity = min(ret_buf.shape[0], ret_meta.shape[0])
+        hint = min(capacity, T * cfg.experts_per_token)
         _lib.call("moe_a2a_combine_recv", self._shape_ref, _ptr(ret_buf), _ptr(ret_meta),
-                  _ptr(ret_counts), hint, _ptr(weights), T, _ptr(out_tokens), int(bool(accumulate)),
+                  _ptr(ret_counts), hint, capacity, _ptr(weights), T, _ptr(out_tokens), int(bool(accumulate)),
                   _DT[dtype_name(cfg.out_dtype)], _stream(self.device))
         return out_tokens
 
@@ -227,10 +229,14 @@ class HIPAllToAll:
 
 def exchange_leg(src: HIPAllToAll, dst: HIPAllToAll, send_counts, send_buf, send_meta,
                  recv_counts, recv_buf, recv_meta, rows_hint: int) -> None:
-    """One source->destination leg of an exchange as a device copy."""
+    """One source->destination leg of an exchange as a device copy. The copy stays inside the
+    rows the four buffers were allocated with, whatever the counts say."""
+    send_capacity = min(send_buf.shape[0], send_meta.shape[0])
+    recv_capacity = min(recv_buf.shape[0], recv_meta.shape[0])
     _lib.call("moe_a2a_exchange_local", src.world_size, src.cfg.hidden_dim, _ptr(send_buf),
               _ptr(send_meta), _ptr(send_counts), dst.rank, _ptr(recv_buf), _ptr(recv_meta),
-              _ptr(recv_counts), src.rank, int(rows_hint), _stream(src.device))
+              _ptr(recv_counts), src.rank, int(rows_hint), send_capacity, recv_capacity,
+              _stream(src.device))
 
 
 class LocalWorld:
@@ -256,6 +262,8 @@ class LocalWorld:
             rc.copy_(per_dst[r])
             for s, src in enumerate(self.ranks):
                 hint = host[s][r] if host is not None else min(bound, sent[s][1].shape[0])
+                if host is not None and hint == 0:
+                    continue  # the counts were read back: this leg is known to be empty
                 exchange_leg(src, dst, sent[s][0], sent[s][1], sent[s][2], rc, rb, rm, hint)
             total = sum(host[s][r] for s in range(W)) if host is not None else None
             got.append((rc, rb, rm, total))

@@ -199,10 +199,12 @@ struct Payload {
 // Sum of max(counts[i], 0) over i < n, computed by every wave on its own: the
 // lanes load the counts side by side (one memory round trip instead of n
 // dependent scalar loads) and reduce with the wave butterfly.
-__device__ __forceinline__ int sum_counts(const int* __restrict__ counts, int n) {
+// Every count is also cut to `cap`; callers make sure n * cap fits an int, so
+// the sum cannot wrap whatever the counts hold.
+__device__ __forceinline__ int sum_counts(const int* __restrict__ counts, int n, int cap) {
   const int lane = threadIdx.x & 63;
   int s = 0;
-  for (int i = lane; i < n; i += 64) s += max(counts[i], 0);
+  for (int i = lane; i < n; i += 64) s += min(max(counts[i], 0), cap);
   return __builtin_amdgcn_readfirstlane(wave_sum(s));
 }
 
@@ -527,20 +529,21 @@ __global__ __launch_bounds__(PLAN_BLOCK) void plan_send_kernel(
 // `hint_rows` rows of recv_buf / recv_meta are readable whatever the counts
 // say. A workgroup whose rows lie below that bound issues all its loads before
 // it knows the true row count R (the counts are loaded at the same time) and
-// only the stores wait for R; rows at or past R are loaded and dropped.
+// only the stores wait for R; rows at or past R are loaded and dropped. Counts
+// that add up to more than `capacity_rows` (what the buffers hold) are cut off there.
 
 template <typename V, int NVW>
 __global__ __launch_bounds__(64 * ROWS) void dispatch_recv_kernel(
     const V* __restrict__ recv_buf, const int* __restrict__ recv_meta,
-    const int* __restrict__ recv_counts, int W, int hint_rows, int nle, uint32_t magic,
-    int max_recv, int row_vecs, int chunks, int* __restrict__ expert_num_tokens,
+    const int* __restrict__ recv_counts, int W, int hint_rows, int capacity_rows, int nle,
+    uint32_t magic, int max_recv, int row_vecs, int chunks, int* __restrict__ expert_num_tokens,
     V* __restrict__ expert_x, int* __restrict__ expert_meta) {
   __shared__ int part[2 * ROWS * ROWS];
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const StridedKeys key{recv_meta, META};
 
   if ((int)blockIdx.x < nle) {
-    const int R = sum_counts(recv_counts, W);
+    const int R = min(sum_counts(recv_counts, W, capacity_rows), capacity_rows);
     const int me = blockIdx.x;
     int c = count_keys<64 * ROWS>(R, key, [=](int e, int) { return floormod(e, nle, magic) == me; });
     c = block_sum<ROWS>(c, part);
@@ -594,11 +597,11 @@ __global__ __launch_bounds__(64 * ROWS) void dispatch_recv_kernel(
   // only groups that lie wholly below the bound: their rows can be read as they are
   const int hint_items = hint_rows / ROWS * chunks;
   if (W <= 64 && q < hint_items) {
-    const int my_count = lane < W ? max(recv_counts[lane], 0) : 0;  // in flight with the rows
-    R = move(q, hint_rows, [&] { return wave_sum(my_count); });
+    const int my_count = lane < W ? min(max(recv_counts[lane], 0), capacity_rows) : 0;  // in flight with the rows
+    R = move(q, hint_rows, [&] { return min(wave_sum(my_count), capacity_rows); });
     q += movers;
   } else {
-    R = sum_counts(recv_counts, W);
+    R = min(sum_counts(recv_counts, W, capacity_rows), capacity_rows);
   }
   const int items = (R + ROWS - 1) / ROWS * chunks;
   for (; q < items; q += movers) move(q, R, [&] { return R; });
@@ -748,7 +751,7 @@ template <typename V, int NVW, bool SMALL>
 __global__ __launch_bounds__(64 * ROWS) void combine_send_kernel(
     const V* __restrict__ expert_y, const int* __restrict__ expert_meta,
     const int* __restrict__ expert_num_tokens, int nle, int max_recv, int W, int row_vecs,
-    int chunks, V* __restrict__ send_buf, int* __restrict__ send_meta,
+    int chunks, int capacity_rows, V* __restrict__ send_buf, int* __restrict__ send_meta,
     int* __restrict__ send_counts) {
   __shared__ int part[2 * ROWS * ROWS];
   __shared__ int pre[SMALL ? 1 : MAX_LOCAL_EXPERTS + 1];
@@ -813,7 +816,7 @@ __global__ __launch_bounds__(64 * ROWS) void combine_send_kernel(
     }, cnt);
     const int slot = rows_reduce(cnt, part, parity, wave, lane);
 
-    if (valid) {
+    if (valid && slot < capacity_rows) {
       p.template store<(MOE_A2A_NT_CSEND != 0)>(send_buf + (size_t)slot * row_vecs, base, row_vecs, lane);
       if (c == 0 && lane < META) send_meta[(size_t)slot * META + lane] = m;
     }
@@ -919,8 +922,8 @@ __device__ __forceinline__ void order_pair(int& ra, int& ka, int& rb, int& kb) {
 template <typename V, int DT, int BLK, int NV>
 __global__ __launch_bounds__(BLK) void combine_recv_kernel(
     const V* __restrict__ recv_buf, const int* __restrict__ recv_meta,
-    const int* __restrict__ recv_counts, int W, int hint_rows, const float* __restrict__ weights,
-    int T, int K, int row_vecs, int chunks, V* __restrict__ out, int accumulate) {
+    const int* __restrict__ recv_counts, int W, int hint_rows, int capacity_rows,
+    const float* __restrict__ weights, int T, int K, int row_vecs, int chunks, V* __restrict__ out, int accumulate) {
   constexpr int N = Words<V>::N;
   constexpr int FAST = 8;  // addends ordered in registers
   __shared__ int hit_row[COMBINE_CAP], hit_k[COMBINE_CAP];
@@ -931,7 +934,7 @@ __global__ __launch_bounds__(BLK) void combine_recv_kernel(
   const int tid = threadIdx.x, lane = tid & 63;
   const int kw = min(K, COMBINE_WEIGHTS);
   const bool lanes_hold_counts = W <= 64;
-  const int my_count = lanes_hold_counts && lane < W ? max(recv_counts[lane], 0) : 0;
+  const int my_count = lanes_hold_counts && lane < W ? min(max(recv_counts[lane], 0), capacity_rows) : 0;
   int R = -1;  // not known yet
 
   // rows [lo, hi) of the arriving stream: note the ones addressed to token t
@@ -947,7 +950,7 @@ __global__ __launch_bounds__(BLK) void combine_recv_kernel(
         key[u] = tk[0];
         kk[u] = tk[1];
       }
-      if (R < 0) R = lanes_hold_counts ? wave_sum(my_count) : sum_counts(recv_counts, W);
+      if (R < 0) R = min(lanes_hold_counts ? wave_sum(my_count) : sum_counts(recv_counts, W, capacity_rows), capacity_rows);
 #pragma unroll
       for (int u = 0; u < SCAN_UNROLL; ++u) {
         const int row = b + tid + u * BLK;
@@ -987,7 +990,7 @@ __global__ __launch_bounds__(BLK) void combine_recv_kernel(
       // first item: one batch below the readable bound goes out before R is known
       const int spec = min(hint_rows, SCAN_UNROLL * BLK);
       scan(t, 0, spec);
-      if (R < 0) R = lanes_hold_counts ? wave_sum(my_count) : sum_counts(recv_counts, W);
+      if (R < 0) R = min(lanes_hold_counts ? wave_sum(my_count) : sum_counts(recv_counts, W, capacity_rows), capacity_rows);
       scan(t, spec, R);
     } else {
       scan(t, 0, R);
@@ -1143,11 +1146,13 @@ __global__ __launch_bounds__(BLOCK) void exchange_local_kernel(
     const V* __restrict__ send_buf, const int* __restrict__ send_meta,
     const int* __restrict__ send_counts, int dst_rank, V* __restrict__ recv_buf,
     int* __restrict__ recv_meta, const int* __restrict__ recv_counts, int src_rank, int row_vecs,
-    int chunks) {
+    int chunks, int send_capacity_rows, int recv_capacity_rows) {
   const int tid = threadIdx.x;
-  const int src_off = sum_counts(send_counts, dst_rank);
-  const int dst_off = sum_counts(recv_counts, src_rank);
-  const int n = min(max(send_counts[dst_rank], 0), max(recv_counts[src_rank], 0));
+  const int src_off = sum_counts(send_counts, dst_rank, send_capacity_rows);
+  const int dst_off = sum_counts(recv_counts, src_rank, recv_capacity_rows);
+  int n = min(max(send_counts[dst_rank], 0), max(recv_counts[src_rank], 0));
+  // never past what either buffer holds, whatever the counts claim
+  n = max(min(n, min(send_capacity_rows - src_off, recv_capacity_rows - dst_off)), 0);
   const int items = n * chunks;
   for (int q = blockIdx.x; q < items; q += gridDim.x) {
     const int i = chunks == 1 ? q : q / chunks, c = q - i * chunks;
@@ -1257,6 +1262,11 @@ int launch_status() { return hipGetLastError() == hipSuccess ? MOE_A2A_OK : MOE_
     }                                             \
   } while (0)
 
+// W counts, each cut to `capacity_rows` on the device, must add up inside an int.
+bool counts_fit(long long capacity_rows, int world_size) {
+  return capacity_rows * world_size <= INT_MAX;
+}
+
 // Workgroups of a ranked row move over `rows` rows.
 long long group_items(long long rows, const Geometry& g) {
   return (rows + ROWS - 1) / ROWS * g.wchunks;
@@ -1317,13 +1327,15 @@ int moe_a2a_plan_send(const moe_a2a_shape* s, const int32_t* indices, int32_t nu
 }
 
 int moe_a2a_dispatch_recv(const moe_a2a_shape* s, const void* recv_buf, const int32_t* recv_meta,
-                          const int32_t* recv_counts, int32_t rows_hint,
+                          const int32_t* recv_counts, int32_t rows_hint, int32_t capacity_rows,
                           int32_t* expert_num_tokens, void* expert_x, int32_t* expert_meta,
                           void* stream) {
-  if (!shape_ok(s) || rows_hint < 0 || !recv_counts || !expert_num_tokens || !expert_x ||
-      !expert_meta)
+  if (!shape_ok(s) || rows_hint < 0 || capacity_rows < 0 || !recv_counts || !expert_num_tokens ||
+      !expert_x || !expert_meta)
     return MOE_A2A_EINVAL;
-  if (rows_hint > 0 && (!recv_buf || !recv_meta)) return MOE_A2A_EINVAL;
+  if (!counts_fit(capacity_rows, s->world_size)) return MOE_A2A_EINVAL;
+  if (rows_hint > capacity_rows) rows_hint = capacity_rows;
+  if (capacity_rows > 0 && (!recv_buf || !recv_meta)) return MOE_A2A_EINVAL;
   if (!all_aligned(2, recv_buf, expert_x)) return MOE_A2A_EALIGN;
   const Geometry g = geometry(s, recv_buf, expert_x);
   // the stream can hold at most nle * max_recv rows that fit the expert buffers
@@ -1332,20 +1344,20 @@ int moe_a2a_dispatch_recv(const moe_a2a_shape* s, const void* recv_buf, const in
   hipStream_t st = (hipStream_t)stream;
 #define LAUNCH(V, NVW)                                                                      \
   dispatch_recv_kernel<V, NVW><<<grid, 64 * ROWS, 0, st>>>(                                 \
-      (const V*)recv_buf, recv_meta, recv_counts, s->world_size, rows_hint, g.nle, g.magic,  \
-      g.max_recv, g.row_vecs, g.wchunks, expert_num_tokens, (V*)expert_x, expert_meta)
+      (const V*)recv_buf, recv_meta, recv_counts, s->world_size, rows_hint, capacity_rows,   \
+      g.nle, g.magic, g.max_recv, g.row_vecs, g.wchunks, expert_num_tokens, (V*)expert_x, expert_meta)
   MOE_A2A_FOR_WAVE_KERNEL(g, LAUNCH);
 #undef LAUNCH
   return launch_status();
 }
 
 int moe_a2a_combine_send(const moe_a2a_shape* s, const void* expert_y, const int32_t* expert_meta,
-                         const int32_t* expert_num_tokens, int32_t rows_hint, void* send_buf,
-                         int32_t* send_meta, int32_t* send_counts, void* stream) {
-  if (!shape_ok(s) || rows_hint < 0 || !expert_y || !expert_meta || !expert_num_tokens ||
-      !send_counts)
+                         const int32_t* expert_num_tokens, int32_t rows_hint,
+                         int32_t capacity_rows, void* send_buf, int32_t* send_meta, int32_t* send_counts, void* stream) {
+  if (!shape_ok(s) || rows_hint < 0 || capacity_rows < 0 || !expert_y || !expert_meta ||
+      !expert_num_tokens || !send_counts)
     return MOE_A2A_EINVAL;
-  if (rows_hint > 0 && (!send_buf || !send_meta)) return MOE_A2A_EINVAL;
+  if (capacity_rows > 0 && (!send_buf || !send_meta)) return MOE_A2A_EINVAL;
   if (!all_aligned(2, expert_y, send_buf)) return MOE_A2A_EALIGN;
   const Geometry g = geometry(s, expert_y, send_buf);
   if (g.nle > MAX_LOCAL_EXPERTS) return MOE_A2A_EINVAL;
@@ -1355,7 +1367,7 @@ int moe_a2a_combine_send(const moe_a2a_shape* s, const void* expert_y, const int
 #define LAUNCH_S(V, NVW, SMALL)                                                                \
   combine_send_kernel<V, NVW, SMALL><<<grid, 64 * ROWS, 0, st>>>(                             \
       (const V*)expert_y, expert_meta, expert_num_tokens, g.nle, g.max_recv, s->world_size,    \
-      g.row_vecs, g.wchunks, (V*)send_buf, send_meta, send_counts)
+      g.row_vecs, g.wchunks, capacity_rows, (V*)send_buf, send_meta, send_counts)
 #define LAUNCH(V, NVW)                        \
   do {                                        \
     if (g.nle <= 64) LAUNCH_S(V, NVW, true);  \
@@ -1368,12 +1380,14 @@ int moe_a2a_combine_send(const moe_a2a_shape* s, const void* expert_y, const int
 }
 
 int moe_a2a_combine_recv(const moe_a2a_shape* s, const void* recv_buf, const int32_t* recv_meta,
-                         const int32_t* recv_counts, int32_t rows_hint, const float* weights,
-                         int32_t num_tokens, void* out_tokens, int32_t accumulate, int32_t dtype,
-                         void* stream) {
+                         const int32_t* recv_counts, int32_t rows_hint, int32_t capacity_rows,
+                         const float* weights, int32_t num_tokens, void* out_tokens,
+                         int32_t accumulate, int32_t dtype, void* stream) {
   if (!shape_ok(s) || num_tokens < 0 || num_tokens > s->max_num_tokens || !recv_counts ||
-      rows_hint < 0)
+      rows_hint < 0 || capacity_rows < 0)
     return MOE_A2A_EINVAL;
+  if (!counts_fit(capacity_rows, s->world_size)) return MOE_A2A_EINVAL;
+  if (rows_hint > capacity_rows) rows_hint = capacity_rows;
   if (dtype != MOE_A2A_F16 && dtype != MOE_A2A_BF16) return MOE_A2A_EINVAL;
   if (num_tokens == 0) return MOE_A2A_OK;
   if (!recv_buf || !recv_meta || !weights || !out_tokens) return MOE_A2A_EINVAL;
@@ -1395,8 +1409,8 @@ int moe_a2a_combine_recv(const moe_a2a_shape* s, const void* recv_buf, const int
   const int K = s->experts_per_token, W = s->world_size;
 #define LAUNCH(V, DT, BLK, NV)                                                               \
   combine_recv_kernel<V, DT, BLK, NV><<<grid, BLK, 0, st>>>(                                 \
-      (const V*)recv_buf, recv_meta, recv_counts, W, rows_hint, weights, num_tokens, K,      \
-      g.row_vecs, chunks, (V*)out_tokens, accumulate)
+      (const V*)recv_buf, recv_meta, recv_counts, W, rows_hint, capacity_rows, weights,      \
+      num_tokens, K, g.row_vecs, chunks, (V*)out_tokens, accumulate)
 #define PICK_SHAPE(V, DT)                       \
   do {                                          \
     if (nv == 1) { LAUNCH(V, DT, BLOCK, 1); }   \
@@ -1453,11 +1467,14 @@ int moe_a2a_expert_scale(const moe_a2a_shape* s, const void* expert_x,
 int moe_a2a_exchange_local(int32_t world_size, int32_t hidden_dim, const void* send_buf,
                            const int32_t* send_meta, const int32_t* send_counts, int32_t dst_rank,
                            void* recv_buf, int32_t* recv_meta, const int32_t* recv_counts,
-                           int32_t src_rank, int32_t rows_hint, void* stream) {
+                           int32_t src_rank, int32_t rows_hint, int32_t send_capacity_rows,
+                           int32_t recv_capacity_rows, void* stream) {
   if (world_size < 1 || hidden_dim < 1 || dst_rank < 0 || dst_rank >= world_size ||
-      src_rank < 0 || src_rank >= world_size || rows_hint < 0 || !send_counts || !recv_counts)
+      src_rank < 0 || src_rank >= world_size || rows_hint < 0 || send_capacity_rows < 0 ||
+      recv_capacity_rows < 0 || !send_counts || !recv_counts ||
+      !counts_fit(send_capacity_rows, world_size) || !counts_fit(recv_capacity_rows, world_size))
     return MOE_A2A_EINVAL;
-  if (rows_hint == 0) return MOE_A2A_OK;
+  if (send_capacity_rows == 0 || recv_capacity_rows == 0) return MOE_A2A_OK;  // nothing can move
   if (!send_buf || !send_meta || !recv_buf || !recv_meta) return MOE_A2A_EINVAL;
   if (!all_aligned(2, send_buf, recv_buf)) return MOE_A2A_EALIGN;
   Geometry g{};
@@ -1468,7 +1485,7 @@ int moe_a2a_exchange_local(int32_t world_size, int32_t hidden_dim, const void* s
 #define LAUNCH(V, NV)                                                                         \
   exchange_local_kernel<V, NV><<<grid, BLOCK, 0, st>>>(                                       \
       (const V*)send_buf, send_meta, send_counts, dst_rank, (V*)recv_buf, recv_meta,          \
-      recv_counts, src_rank, g.row_vecs, g.chunks)
+      recv_counts, src_rank, g.row_vecs, g.chunks, send_capacity_rows, recv_capacity_rows)
   MOE_A2A_FOR_ROW_KERNEL(g, LAUNCH);
 #undef LAUNCH
   return launch_status();

@@ -17,10 +17,14 @@
  *   - every `rows_hint` is a host-side guess of the number of rows the call
  *     will move. Kernels read the true row count from device memory and
  *     stride over it, so a hint that is too small or too large costs time,
- *     never correctness. One rule comes with it: the input row and meta
- *     buffers of the call must be readable for `rows_hint` rows (pass at most
- *     the capacity they were allocated with). Rows between the true count and
- *     the hint may be read before the count is known; they are never used;
+ *     never correctness;
+ *   - every `*capacity_rows` is the number of rows the named row buffer and
+ *     its meta buffer were allocated with. No kernel reads or writes a row at
+ *     or past it, whatever the device-side counts claim: counts that add up
+ *     to more are cut off there (the reference would raise an index error).
+ *     Rows between the true count and min(rows_hint, capacity) may be read
+ *     before the count is known; they are never used. capacity * world_size
+ *     must fit an int32 (MOE_A2A_EINVAL beyond);
  *   - return value: MOE_A2A_OK (0) or a negative MOE_A2A_E* code. Argument
  *     errors are detected before anything is launched.
  *
@@ -118,6 +122,7 @@ int moe_a2a_plan_send(const moe_a2a_shape* shape, const int32_t* indices,
  *                       segment first, each in the sender's order
  *   recv_meta   [R, 5]
  *   recv_counts [W] int32, rows received from each source rank; R = their sum
+ *   capacity_rows       rows recv_buf / recv_meta were allocated with
  *   expert_num_tokens [nle] int32 out (every entry written, zeros included)
  *   expert_x    [nle, max_recv, H] out; only rows < expert_num_tokens[le] are
  *                       written (the reference leaves the rest uninitialised
@@ -128,8 +133,9 @@ int moe_a2a_plan_send(const moe_a2a_shape* shape, const int32_t* indices,
  */
 int moe_a2a_dispatch_recv(const moe_a2a_shape* shape, const void* recv_buf,
                           const int32_t* recv_meta, const int32_t* recv_counts,
-                          int32_t rows_hint, int32_t* expert_num_tokens,
-                          void* expert_x, int32_t* expert_meta, void* stream);
+                          int32_t rows_hint, int32_t capacity_rows,
+                          int32_t* expert_num_tokens, void* expert_x,
+                          int32_t* expert_meta, void* stream);
 
 /*
  * Combine, send side: expert-major results -> rows grouped by origin rank.
@@ -138,14 +144,16 @@ int moe_a2a_dispatch_recv(const moe_a2a_shape* shape, const void* recv_buf,
  *
  *   expert_y    [nle, max_recv, H], expert_meta [nle, max_recv, 5],
  *   expert_num_tokens [nle] (values above max_recv are clamped)
- *   send_buf    [R, H] out, send_meta [R, 5] out (meta rows copied unchanged)
+ *   send_buf    [R, H] out, send_meta [R, 5] out (meta rows copied unchanged);
+ *               capacity_rows is their allocation
  *   send_counts [W] int32 out
  */
 int moe_a2a_combine_send(const moe_a2a_shape* shape, const void* expert_y,
                          const int32_t* expert_meta,
                          const int32_t* expert_num_tokens, int32_t rows_hint,
-                         void* send_buf, int32_t* send_meta,
-                         int32_t* send_counts, void* stream);
+                         int32_t capacity_rows, void* send_buf,
+                         int32_t* send_meta, int32_t* send_counts,
+                         void* stream);
 
 /*
  * Combine, receive side: weighted sum back into token order.
@@ -169,9 +177,10 @@ int moe_a2a_combine_send(const moe_a2a_shape* shape, const void* expert_y,
  */
 int moe_a2a_combine_recv(const moe_a2a_shape* shape, const void* recv_buf,
                          const int32_t* recv_meta, const int32_t* recv_counts,
-                         int32_t rows_hint, const float* weights,
-                         int32_t num_tokens, void* out_tokens,
-                         int32_t accumulate, int32_t dtype, void* stream);
+                         int32_t rows_hint, int32_t capacity_rows,
+                         const float* weights, int32_t num_tokens,
+                         void* out_tokens, int32_t accumulate, int32_t dtype,
+                         void* stream);
 
 /*
  * Stand-in for the expert computation between dispatch and combine.
@@ -202,7 +211,8 @@ int moe_a2a_exchange_local(int32_t world_size, int32_t hidden_dim,
                            const int32_t* send_counts, int32_t dst_rank,
                            void* recv_buf, int32_t* recv_meta,
                            const int32_t* recv_counts, int32_t src_rank,
-                           int32_t rows_hint, void* stream);
+                           int32_t rows_hint, int32_t send_capacity_rows,
+                           int32_t recv_capacity_rows, void* stream);
 
 #ifdef __cplusplus
 }

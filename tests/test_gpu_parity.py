@@ -405,3 +405,100 @@ def test_random_small_jobs():
                     dtype=str(rng.choice(["bf16", "fp16"])))
         print(f"random job {case}: {spec}", flush=True)
         run_and_compare(generate_world(spec, 9000 + case), exact_hints=bool(case % 2))
+
+
+def test_counts_beyond_capacity_are_cut_off():
+    """Device-side counts that claim more rows than the caller says its buffers hold: every
+    kernel stops at the stated capacity. The tensors here are really allocated with 64 rows and
+    pre-filled with a sentinel, the calls are told 24 (or 40), and nothing past that may be read
+    into a result or written."""
+    import ctypes as C
+    from amd_distributed_2025_amd import HIPAllToAll, _lib
+
+    W, nle, K, H, max_T = 4, 2, 2, 72, 8
+    cfg = MoEConfig(W * nle, K, H, max_T, in_dtype=torch.bfloat16, out_dtype=torch.bfloat16)
+    a = HIPAllToAll(cfg, 0, W, device=DEV)
+    max_recv = max_T * W
+    rng = np.random.default_rng(77)
+    ALLOC, CAP, SENT = 64, 24, -12345
+    p = lambda t: C.c_void_p(t.data_ptr())
+    st = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    shape = C.byref(a.shape)
+
+    def rows(n):
+        return torch.from_numpy(rng.integers(0, 0x4400, (n, H), dtype=np.int16)).view(torch.bfloat16).to(DEV)
+
+    # ---- dispatch_recv: counts claim 40 rows, the buffers are said to hold 24
+    meta_np = np.zeros((ALLOC, 5), np.int32)
+    meta_np[:, 0] = rng.integers(0, nle, ALLOC)
+    meta_np[:, 1] = np.repeat(np.arange(W), ALLOC // W)
+    meta_np[:, 2] = rng.integers(0, max_T, ALLOC)
+    meta_np[:, 3] = rng.integers(0, K, ALLOC)
+    recv_buf, recv_meta = rows(ALLOC), torch.from_numpy(meta_np).to(DEV)
+    counts40 = torch.tensor([10, 10, 10, 10], dtype=torch.int32, device=DEV)
+    num = torch.full((nle,), SENT, dtype=torch.int32, device=DEV)
+    ex = torch.zeros(nle, max_recv, H, dtype=torch.bfloat16, device=DEV)
+    em = torch.full((nle, max_recv, 5), SENT, dtype=torch.int32, device=DEV)
+    for hint in (0, 7, CAP, 40, 1000):
+        num.fill_(SENT); em.fill_(SENT)
+        _lib.call("moe_a2a_dispatch_recv", shape, p(recv_buf), p(recv_meta), p(counts40), hint, CAP,
+                  p(num), p(ex), p(em), st)
+        torch.cuda.synchronize()
+        cnt, local, pos, order = orc.expert_placement(meta_np[:CAP], nle)
+        assert np.array_equal(num.cpu().numpy(), cnt), hint
+        assert np.array_equal(valid_rows(em, cnt).numpy(), meta_np[:CAP][order]), hint
+        assert np.array_equal(bits(valid_rows(ex, cnt)), bits(recv_buf[:CAP])[order]), hint
+        for le in range(nle):
+            assert bool((em[le, int(cnt[le]):] == SENT).all()), hint
+
+    # ---- combine_send: the experts hold 40 rows, the send buffers are said to hold 24
+    cnt40, _, _, order40 = orc.expert_placement(meta_np[:40], nle)
+    ey = torch.zeros(nle, max_recv, H, dtype=torch.bfloat16, device=DEV)
+    em.fill_(SENT)
+    stream_meta = meta_np[:40][order40]
+    stream_rows = rows(40)
+    at = 0
+    for le in range(nle):
+        n = int(cnt40[le])
+        ey[le, :n] = stream_rows[at:at + n]
+        em[le, :n] = torch.from_numpy(stream_meta[at:at + n]).to(DEV)
+        at += n
+    num40 = torch.from_numpy(cnt40).to(DEV)
+    back_buf = torch.zeros(ALLOC, H, dtype=torch.bfloat16, device=DEV)
+    back_meta = torch.full((ALLOC, 5), SENT, dtype=torch.int32, device=DEV)
+    back_counts = torch.full((W,), SENT, dtype=torch.int32, device=DEV)
+    for hint in (0, CAP, 40, 1000):
+        back_meta.fill_(SENT); back_buf.zero_()
+        _lib.call("moe_a2a_combine_send", shape, p(ey), p(em), p(num40), hint, CAP, p(back_buf),
+                  p(back_meta), p(back_counts), st)
+        torch.cuda.synchronize()
+        bc, bo = orc.return_order(stream_meta, W)
+        assert np.array_equal(back_counts.cpu().numpy(), bc), hint   # counts are the true ones
+        assert np.array_equal(back_meta.cpu().numpy()[:CAP], stream_meta[bo][:CAP]), hint
+        assert np.array_equal(bits(back_buf[:CAP]), bits(stream_rows)[bo][:CAP]), hint
+        assert bool((back_meta[CAP:] == SENT).all()) and not bool(back_buf[CAP:].any()), hint
+
+    # ---- exchange leg: the source's segment for rank 1 starts at row 30 of a buffer said to hold 40
+    send_counts = torch.tensor([30, 30, 0, 0], dtype=torch.int32, device=DEV)
+    recv_counts = torch.tensor([30, 30, 0, 0], dtype=torch.int32, device=DEV)
+    dst_buf = torch.zeros(ALLOC, H, dtype=torch.bfloat16, device=DEV)
+    dst_meta = torch.full((ALLOC, 5), SENT, dtype=torch.int32, device=DEV)
+    for send_cap, recv_cap, moved in ((40, ALLOC, 10), (ALLOC, 5, 5), (ALLOC, ALLOC, 30), (20, ALLOC, 0)):
+        dst_buf.zero_(); dst_meta.fill_(SENT)
+        # source rank 0 -> destination rank 1: reads rows [30, 60) of the source, writes rows [0, 30)
+        _lib.call("moe_a2a_exchange_local", W, H, p(recv_buf), p(recv_meta), p(send_counts), 1,
+                  p(dst_buf), p(dst_meta), p(recv_counts), 0, 30, send_cap, recv_cap, st)
+        torch.cuda.synchronize()
+        assert torch.equal(dst_buf[:moved], recv_buf[30:30 + moved]), (send_cap, recv_cap)
+        assert torch.equal(dst_meta[:moved], recv_meta[30:30 + moved]), (send_cap, recv_cap)
+        assert bool((dst_meta[moved:] == SENT).all()) and not bool(dst_buf[moved:].any()), (send_cap, recv_cap)
+
+    # ---- combine_recv: counts claim 40 arrivals, the buffers are said to hold 24
+    weights = torch.from_numpy(rng.random((max_T, K), dtype=np.float32)).to(DEV)
+    y = torch.zeros(max_T, H, dtype=torch.bfloat16, device=DEV)
+    for hint in (0, CAP, 40, 1000):
+        _lib.call("moe_a2a_combine_recv", shape, p(recv_buf), p(recv_meta), p(counts40), hint, CAP,
+                  p(weights), max_T, p(y), 0, _lib.BF16, st)
+        torch.cuda.synchronize()
+        want = orc.combine_recv(bits(recv_buf[:CAP]), meta_np[:CAP], weights.cpu().numpy(), max_T, "bf16")
+        assert np.array_equal(bits(y), want), hint
