@@ -182,12 +182,16 @@ struct Payload {
 #pragma unroll
     for (int j = 0; j < NV; ++j) v[j] = stream_load(row + min(base + j * BLOCK + (int)threadIdx.x, row_vecs - 1));
   }
-  __device__ __forceinline__ void store(V* __restrict__ row, int base, int row_vecs) const {
+  template <bool NT>
+  __device__ __forceinline__ void store_as(V* __restrict__ row, int base, int row_vecs) const {
 #pragma unroll
     for (int j = 0; j < NV; ++j) {
       const int idx = base + j * BLOCK + threadIdx.x;
-      if (idx < row_vecs) row_store<(MOE_A2A_NT_STANDIN != 0)>(row + idx, v[j]);
+      if (idx < row_vecs) row_store<NT>(row + idx, v[j]);
     }
+  }
+  __device__ __forceinline__ void store(V* __restrict__ row, int base, int row_vecs) const {
+    store_as<(MOE_A2A_NT_STANDIN != 0)>(row, base, row_vecs);
   }
   template <typename F>
   __device__ __forceinline__ void map(F f) {
@@ -399,6 +403,109 @@ __global__ __launch_bounds__(64 * ROWS) void dispatch_send_kernel(
           send_meta[(size_t)slot * META + lane] = m;
         }
         if (lane == 0 && send_slot) send_slot[i] = slot;
+      }
+    }
+  }
+}
+
+// Stage 1 with one workgroup per (token, row chunk): the token's row is loaded
+// once, its K entries are ranked together (FAN at a time) in one pass over the
+// keys, and the row held in registers is stored to each of their slots. Compared
+// with a wave per entry this reads every source row once instead of K times and
+// issues an eighth of the key loads. The order is carried by one composite key
+// per entry, class * S + i with class = 0 (id < 0), 1 + destination, W + 1
+// (id >= E): entry a precedes entry b exactly when its composite key is smaller.
+// The host uses this kernel when (W + 2) * S fits an int.
+
+constexpr int FAN = 8;
+
+template <typename V, int NV>
+__global__ __launch_bounds__(BLOCK) void dispatch_fanout_kernel(
+    const V* __restrict__ x, const int* __restrict__ indices, int T, int K, int nle, int E, int W,
+    uint32_t magic, int rank, int row_vecs, int chunks, V* __restrict__ send_buf,
+    int* __restrict__ send_meta, int* __restrict__ send_counts, int* __restrict__ send_slot) {
+  __shared__ int part[2 * NWAVES * FAN];
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int S = T * K;
+  auto klass = [&](int e) {
+    return e < 0 ? 0 : e >= E ? W + 1 : 1 + (nle == 1 ? e : (int)__umulhi((uint32_t)e, magic));
+  };
+
+  if ((int)blockIdx.x < W) {
+    const int want = blockIdx.x + 1;
+    int c = count_keys<BLOCK>(S, StridedKeys{indices, 1}, [&](int e, int) { return klass(e) == want; });
+    c = block_sum<NWAVES>(c, part);
+    if (tid == 0) send_counts[blockIdx.x] = c;
+    return;
+  }
+
+  const int items = T * chunks, movers = gridDim.x - W;
+  int parity = 0;
+  for (int q = blockIdx.x - W; q < items; q += movers) {
+    const int t = chunks == 1 ? q : q / chunks, c = q - t * chunks;
+    const int base = c * (BLOCK * NV);
+    const int i0 = t * K;
+
+    // first batch of keys, then the row: the keys come back first
+    int key[SCAN_UNROLL];
+#pragma unroll
+    for (int u = 0; u < SCAN_UNROLL; ++u) key[u] = indices[min(tid + u * BLOCK, S - 1)];
+    Payload<V, NV> p;
+    p.load(x + (size_t)t * row_vecs, base, row_vecs);
+
+    for (int g0 = 0; g0 < K; g0 += FAN) {
+      int mine[FAN];
+#pragma unroll
+      for (int g = 0; g < FAN; ++g) {
+        const int i = i0 + min(g0 + g, K - 1);
+        mine[g] = klass(indices[i]) * S + i;
+      }
+      int cnt[FAN];
+#pragma unroll
+      for (int g = 0; g < FAN; ++g) cnt[g] = 0;
+      auto consume = [&](const int (&k)[SCAN_UNROLL], int b) {
+#pragma unroll
+        for (int u = 0; u < SCAN_UNROLL; ++u) {
+          const int i2 = b + tid + u * BLOCK;
+          const int ck = i2 < S ? klass(k[u]) * S + i2 : INT_MAX;
+#pragma unroll
+          for (int g = 0; g < FAN; ++g) cnt[g] += (int)(ck < mine[g]);
+        }
+      };
+      consume(key, 0);
+      for (int b = SCAN_UNROLL * BLOCK; b < S; b += SCAN_UNROLL * BLOCK) {
+        int more[SCAN_UNROLL];
+#pragma unroll
+        for (int u = 0; u < SCAN_UNROLL; ++u) more[u] = indices[min(b + tid + u * BLOCK, S - 1)];
+        consume(more, b);
+      }
+
+      int* half = part + (parity++ & 1) * (NWAVES * FAN);
+#pragma unroll
+      for (int g = 0; g < FAN; ++g) {
+        const int sum = wave_sum(cnt[g]);
+        if (lane == 0) half[wave * FAN + g] = sum;
+      }
+      lds_barrier();
+      const int live = min(FAN, K - g0);
+#pragma unroll
+      for (int g = 0; g < FAN; ++g) {
+        if (g < live) {
+          int slot = 0;
+#pragma unroll
+          for (int w = 0; w < NWAVES; ++w) slot += half[w * FAN + g];
+          p.template store_as<(MOE_A2A_NT_SEND != 0)>(send_buf + (size_t)slot * row_vecs, base, row_vecs);
+        }
+      }
+      if (c == 0 && tid < live * META) {
+        const int g = tid / META, f = tid - g * META;
+        int slot = 0;
+#pragma unroll
+        for (int w = 0; w < NWAVES; ++w) slot += half[w * FAN + g];
+        const int i = i0 + g0 + g;
+        const int m = f == 0 ? indices[i] : f == 1 ? rank : f == 2 ? t : f == 3 ? g0 + g : 0;
+        send_meta[(size_t)slot * META + f] = m;
+        if (f == 0 && send_slot) send_slot[i] = slot;
       }
     }
   }
@@ -1298,8 +1405,30 @@ int moe_a2a_dispatch_send(const moe_a2a_shape* s, const void* x, const int32_t* 
   if (!all_aligned(2, x, send_buf)) return MOE_A2A_EALIGN;
   const Geometry g = geometry(s, x, send_buf);
   if (!items_fit(S, g.wchunks)) return MOE_A2A_EINVAL;
-  const int grid = s->world_size + mover_blocks(group_items(S, g));
   hipStream_t st = (hipStream_t)stream;
+  // Tokens with several entries: one workgroup per (token, 256-vector chunk) stores the chunk to
+  // all of the token's slots (measured at K = 8, H = 7168: 8.4 us against 8.8 us with a wave per
+  // entry; one chunk per workgroup beats two or four). With one or two entries per token the
+  // wave-per-entry kernel scans fewer keys per byte moved.
+#ifndef MOE_A2A_FANOUT_MIN_K
+#define MOE_A2A_FANOUT_MIN_K 4
+#endif
+  Geometry f = g;
+  f.nv = 1;
+  f.chunks = (f.row_vecs + BLOCK - 1) / BLOCK;
+  if (s->experts_per_token >= MOE_A2A_FANOUT_MIN_K && (s->world_size + 2ll) * S <= INT_MAX &&
+      items_fit(num_tokens, f.chunks)) {
+    const int fgrid = s->world_size + mover_blocks((long long)num_tokens * f.chunks);
+#define LAUNCH(V, NV)                                                                          \
+  dispatch_fanout_kernel<V, NV><<<fgrid, BLOCK, 0, st>>>(                                      \
+      (const V*)x, indices, num_tokens, s->experts_per_token, g.nle, s->num_experts,           \
+      s->world_size, g.magic, s->rank, f.row_vecs, f.chunks, (V*)send_buf, send_meta,          \
+      send_counts, send_slot)
+    MOE_A2A_FOR_ROW_KERNEL(f, LAUNCH);
+#undef LAUNCH
+    return launch_status();
+  }
+  const int grid = s->world_size + mover_blocks(group_items(S, g));
 #define LAUNCH(V, NVW)                                                                         \
   dispatch_send_kernel<V, NVW><<<grid, 64 * ROWS, 0, st>>>(                                    \
       (const V*)x, indices, (int)S, s->experts_per_token, g.nle, s->num_experts, s->world_size, \

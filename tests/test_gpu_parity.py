@@ -135,6 +135,8 @@ EDGE = {
                        max_num_tokens=7, num_tokens="full", dtype="fp16"),
     "wide_rows_two_chunks": dict(world_size=2, num_experts=4, experts_per_token=2, hidden_dim=16384,
                                  max_num_tokens=6, num_tokens="full", dtype="bf16"),
+    "many_entries_several_key_batches": dict(world_size=2, num_experts=16, experts_per_token=10, hidden_dim=64,
+                                             max_num_tokens=300, num_tokens="full", dtype="bf16"),
     "k_above_fast_list": dict(world_size=2, num_experts=160, experts_per_token=72, hidden_dim=64,
                               max_num_tokens=3, num_tokens="full", dtype="bf16"),
 }
