@@ -40,8 +40,8 @@ _SP = C.POINTER(Shape)
 SIGNATURES = {
     "moe_a2a_dispatch_send": [_SP, _P, _P, _I, _P, _P, _P, _P, _P],
     "moe_a2a_plan_send": [_SP, _P, _I, _P, _P, _P, _P, _P, _P],
-    "moe_a2a_dispatch_recv": [_SP, _P, _P, _P, _I, _I, _P, _P, _P, _P],
-    "moe_a2a_combine_send": [_SP, _P, _P, _P, _I, _I, _P, _P, _P, _P],
+    "moe_a2a_dispatch_recv": [_SP, _P, _P, _P, _I, _I, _P, _P, _P, _P, _P],
+    "moe_a2a_combine_send": [_SP, _P, _P, _P, _I, _I, _P, _P, _P, _P, _P],
     "moe_a2a_combine_recv": [_SP, _P, _P, _P, _I, _I, _P, _I, _P, _I, _I, _P],
     "moe_a2a_expert_scale": [_SP, _P, _P, _I, _I, _I, _P, _P],
     "moe_a2a_exchange_local": [_I, _I, _P, _P, _P, _I, _P, _P, _P, _I, _I, _I, _I, _P],

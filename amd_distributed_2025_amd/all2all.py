@@ -51,7 +51,8 @@ def _need(t: torch.Tensor, dtype: torch.dtype, device, what: str) -> torch.Tenso
 class HIPAllToAll:
     META_DIM = META_DIM  # global_exp, src_rank, src_token, src_k, pad
 
-    def __init__(self, cfg: MoEConfig, rank: int, world_size: int, exchange=None, device=None):
+    def __init__(self, cfg: MoEConfig, rank: int, world_size: int, exchange=None, device=None,
+                 reuse_placement: bool = True):
         if cfg.num_experts % world_size:
             raise ValueError("num_experts must be a multiple of world_size")
         self.cfg = cfg
@@ -71,6 +72,10 @@ class HIPAllToAll:
         self.max_rows_in = self.max_recv * min(cfg.experts_per_token, self.num_local_experts)
         self.max_rows_out = cfg.max_num_tokens * cfg.experts_per_token
         self._ws = {}
+        # dispatch_recv leaves a plan of where combine_send will put every row; combine_send uses
+        # it when it is handed the very tensors that dispatch_recv returned
+        self.reuse_placement = reuse_placement
+        self._planned_for = None
 
     # ------------------------------------------------------------------ workspace
 
@@ -147,8 +152,11 @@ class HIPAllToAll:
         num = self._buf("expert_num_tokens", (nle,), torch.int32)
         ex = self._buf("expert_x", (nle, self.max_recv, cfg.hidden_dim), cfg.in_dtype)
         em = self._buf("expert_meta", (nle, self.max_recv, META_DIM), torch.int32)
+        plan = self._buf("send_back_plan", (2 * cfg.num_experts,), torch.int32) if self.reuse_placement else None
         _lib.call("moe_a2a_dispatch_recv", self._shape_ref, _ptr(recv_buf), _ptr(recv_meta),
-                  _ptr(recv_counts), hint, capacity, _ptr(num), _ptr(ex), _ptr(em), _stream(self.device))
+                  _ptr(recv_counts), hint, capacity, _ptr(num), _ptr(ex), _ptr(em), _ptr(plan),
+                  _stream(self.device))
+        self._planned_for = None if plan is None else (em.data_ptr(), num.data_ptr())
         self._rows_in_hint = hint
         return num, ex, em
 
@@ -178,9 +186,15 @@ class HIPAllToAll:
         counts = self._buf("back_counts", (self.world_size,), torch.int32)
         buf = self._buf("back_buf", (self.max_rows_in, cfg.hidden_dim), cfg.out_dtype)
         meta = self._buf("back_meta", (self.max_rows_in, META_DIM), torch.int32)
+        # the plan describes expert_meta / expert_num_tokens as dispatch_recv wrote them: a caller
+        # that edits them in place between the two calls must build the object with
+        # reuse_placement=False
+        plan = None
+        if self._planned_for == (expert_meta.data_ptr(), expert_num_tokens.data_ptr()):
+            plan = self._ws["send_back_plan"]
         _lib.call("moe_a2a_combine_send", self._shape_ref, _ptr(expert_y), _ptr(expert_meta),
                   _ptr(expert_num_tokens), min(hint, self.max_rows_in), self.max_rows_in, _ptr(buf),
-                  _ptr(meta), _ptr(counts), _stream(self.device))
+                  _ptr(meta), _ptr(counts), _ptr(plan), _stream(self.device))
         return counts, buf, meta
 
     def combine_recv(self, out_tokens, weights, ret_counts, ret_buf, ret_meta, accumulate: bool = True):
@@ -243,9 +257,11 @@ class LocalWorld:
     """All ranks of one job on one GPU, stepped in lockstep; the exchanges are
     device copies (stand-in for all2all/reference.py:91,107-119,185,210-222)."""
 
-    def __init__(self, cfg: MoEConfig, world_size: int, device=None, exact_hints: bool = True):
+    def __init__(self, cfg: MoEConfig, world_size: int, device=None, exact_hints: bool = True,
+                 reuse_placement: bool = True):
         self.cfg, self.world_size = cfg, world_size
-        self.ranks = [HIPAllToAll(cfg, r, world_size, device=device) for r in range(world_size)]
+        self.ranks = [HIPAllToAll(cfg, r, world_size, device=device, reuse_placement=reuse_placement)
+                      for r in range(world_size)]
         self.device = self.ranks[0].device
         self.exact_hints = exact_hints  # read the counts back to size the copies exactly
         self.trace: List[dict] = [dict() for _ in range(world_size)]

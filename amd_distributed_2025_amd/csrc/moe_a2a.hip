@@ -639,15 +639,73 @@ __global__ __launch_bounds__(PLAN_BLOCK) void plan_send_kernel(
 // only the stores wait for R; rows at or past R are loaded and dropped. Counts
 // that add up to more than `capacity_rows` (what the buffers hold) are cut off there.
 
-template <typename V, int NVW>
+//
+// PLAN (W <= 64): the counting workgroup of expert le also splits its rows by
+// source rank and writes, for every source s, two ints at plan[(le*W + s)*2]:
+//   [0] the position inside expert le at which the rows from s start (inside an
+//       expert, rows lie in arrival order, that is by source rank), and
+//   [1] the row of the send-back stream of stage 3 that the first of them goes
+//       to: #{rows from lower sources} + #{rows from s in lower experts}.
+// Stage 3 then places a row without scanning any keys.
+
+constexpr int PLAN_INTS = 2;  // ints per (local expert, source rank) of the send-back plan
+
+template <typename V, int NVW, bool PLAN>
 __global__ __launch_bounds__(64 * ROWS) void dispatch_recv_kernel(
     const V* __restrict__ recv_buf, const int* __restrict__ recv_meta,
     const int* __restrict__ recv_counts, int W, int hint_rows, int capacity_rows, int nle,
     uint32_t magic, int max_recv, int row_vecs, int chunks, int* __restrict__ expert_num_tokens,
-    V* __restrict__ expert_x, int* __restrict__ expert_meta) {
+    V* __restrict__ expert_x, int* __restrict__ expert_meta, int* __restrict__ plan) {
   __shared__ int part[2 * ROWS * ROWS];
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const StridedKeys key{recv_meta, META};
+
+  if constexpr (PLAN) {
+    if ((int)blockIdx.x < nle) {
+      __shared__ int seg_end[64];  // rows received from sources 0..s
+      __shared__ int hist[64][2];  // per source: rows of this expert, rows of lower experts
+      const int me = blockIdx.x;
+      const int mine = lane < W ? min(max(recv_counts[lane], 0), capacity_rows) : 0;
+      const int incl = wave_inclusive_scan(mine);
+      const int R = min(__builtin_amdgcn_readlane(incl, 63), capacity_rows);
+      if (wave == 0 && lane < W) {
+        seg_end[lane] = incl;
+        hist[lane][0] = 0;
+        hist[lane][1] = 0;
+      }
+      lds_barrier();
+      constexpr int BLK = 64 * ROWS;
+      for (int b = 0; b < R; b += SCAN_UNROLL * BLK) {
+        int e2[SCAN_UNROLL];
+#pragma unroll
+        for (int u = 0; u < SCAN_UNROLL; ++u)
+          e2[u] = recv_meta[(size_t)min(b + tid + u * BLK, R - 1) * META];
+#pragma unroll
+        for (int u = 0; u < SCAN_UNROLL; ++u) {
+          const int i2 = b + tid + u * BLK;
+          const int le2 = floormod(e2[u], nle, magic);
+          if (i2 < R && le2 <= me) {
+            int src = 0;
+            for (int s = 0; s + 1 < W; ++s) src += (int)(seg_end[s] <= i2);
+            atomicAdd(&hist[src][le2 < me ? 1 : 0], 1);
+          }
+        }
+      }
+      lds_barrier();
+      if (wave == 0) {
+        const int here = lane < W ? hist[lane][0] : 0;
+        const int below = lane < W ? hist[lane][1] : 0;
+        const int upto = wave_inclusive_scan(here);
+        if (lane < W) {
+          int* out = plan + ((size_t)me * W + lane) * PLAN_INTS;
+          out[0] = upto - here;
+          out[1] = (incl - mine) + below;
+        }
+        if (lane == 63) expert_num_tokens[me] = upto;
+      }
+      return;
+    }
+  }
 
   if ((int)blockIdx.x < nle) {
     const int R = min(sum_counts(recv_counts, W, capacity_rows), capacity_rows);
@@ -854,15 +912,70 @@ struct WaveStreamKeys {
 // order. Row g with origin d goes to slot
 //   #{rows of a lower origin} + #{earlier rows of origin d}.
 
-template <typename V, int NVW, bool SMALL>
+//
+// PLAN (needs SMALL and W <= 64): stage 2 left, for every (local expert, source
+// rank), where that run of rows starts inside the expert and in the send-back
+// stream (see dispatch_recv_kernel). A wave then finds the run its row lies in
+// with one ballot over W lanes and needs no key scan and no exchange with the
+// other waves. The plan counts every received row, so it only describes the
+// buffers when no expert overflowed max_recv; if one did, every workgroup sees
+// it in the counts and takes the scan instead.
+
+template <typename V, int NVW, bool SMALL, bool PLAN>
 __global__ __launch_bounds__(64 * ROWS) void combine_send_kernel(
     const V* __restrict__ expert_y, const int* __restrict__ expert_meta,
     const int* __restrict__ expert_num_tokens, int nle, int max_recv, int W, int row_vecs,
     int chunks, int capacity_rows, V* __restrict__ send_buf, int* __restrict__ send_meta,
-    int* __restrict__ send_counts) {
+    int* __restrict__ send_counts, const int* __restrict__ plan) {
+  static_assert(!PLAN || SMALL, "the planned path keeps the expert prefix in registers");
   __shared__ int part[2 * ROWS * ROWS];
   __shared__ int pre[SMALL ? 1 : MAX_LOCAL_EXPERTS + 1];
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+
+  if constexpr (PLAN) {
+    const int raw = lane < nle ? expert_num_tokens[lane] : 0;
+    if (__ballot(raw > max_recv) == 0) {
+      const int have = max(raw, 0);
+      const int incl = wave_inclusive_scan(have), excl = incl - have;
+      const int R = __builtin_amdgcn_readlane(incl, 63);
+
+      if ((int)blockIdx.x < W) {
+        // rows that go back to origin `me`: the lengths of its runs, one expert per lane
+        const int me = blockIdx.x;
+        int len = 0;
+        if (lane < nle) {
+          const int* run = plan + ((size_t)lane * W + me) * PLAN_INTS;
+          len = (me + 1 < W ? run[PLAN_INTS] : have) - run[0];
+        }
+        const int total = wave_sum(len);
+        if (tid == 0) send_counts[me] = total;
+        return;
+      }
+
+      const int items = R * chunks, movers = (gridDim.x - W) * ROWS;
+      for (int q = (blockIdx.x - W) * ROWS + wave; q < items; q += movers) {
+        const int g = chunks == 1 ? q : q / chunks, c = q - g * chunks;
+        const int base = c * (64 * NVW);
+        const int le = __popcll(__ballot(incl <= g));
+        const int j = g - __builtin_amdgcn_readlane(excl, le);
+        const size_t row = (size_t)le * max_recv + j;
+        int run[PLAN_INTS] = {INT_MAX, 0};
+        if (lane < W) __builtin_memcpy(run, plan + ((size_t)le * W + lane) * PLAN_INTS, sizeof(run));
+        int m = 0;
+        if (c == 0 && lane < META) m = expert_meta[row * META + lane];
+        WavePayload<V, NVW> p;
+        p.load(expert_y + row * row_vecs, base, row_vecs, lane);
+        // the run starts are ascending in the source rank: the last one at or below j is ours
+        const int src = max(__popcll(__ballot(run[0] <= j)) - 1, 0);
+        const int slot = __builtin_amdgcn_readlane(run[1], src) + (j - __builtin_amdgcn_readlane(run[0], src));
+        if (slot >= 0 && slot < capacity_rows) {
+          p.template store<(MOE_A2A_NT_CSEND != 0)>(send_buf + (size_t)slot * row_vecs, base, row_vecs, lane);
+          if (c == 0 && lane < META) send_meta[(size_t)slot * META + lane] = m;
+        }
+      }
+      return;
+    }
+  }
 
   // SMALL (nle <= 64): prefix in registers; otherwise the LDS table
   using Keys = typename std::conditional<SMALL, WaveStreamKeys<1>, ExpertStreamKeys<1>>::type;
@@ -1369,6 +1482,12 @@ int launch_status() { return hipGetLastError() == hipSuccess ? MOE_A2A_OK : MOE_
     }                                             \
   } while (0)
 
+// The send-back plan is kept by the lanes of one wave: one lane per source rank
+// in stage 2, one lane per local expert in stage 3.
+bool plan_supported(const moe_a2a_shape* s) {
+  return s->world_size <= 64 && s->num_experts / s->world_size <= 64;
+}
+
 // W counts, each cut to `capacity_rows` on the device, must add up inside an int.
 bool counts_fit(long long capacity_rows, int world_size) {
   return capacity_rows * world_size <= INT_MAX;
@@ -1458,7 +1577,7 @@ int moe_a2a_plan_send(const moe_a2a_shape* s, const int32_t* indices, int32_t nu
 int moe_a2a_dispatch_recv(const moe_a2a_shape* s, const void* recv_buf, const int32_t* recv_meta,
                           const int32_t* recv_counts, int32_t rows_hint, int32_t capacity_rows,
                           int32_t* expert_num_tokens, void* expert_x, int32_t* expert_meta,
-                          void* stream) {
+                          int32_t* send_back_plan, void* stream) {
   if (!shape_ok(s) || rows_hint < 0 || capacity_rows < 0 || !recv_counts || !expert_num_tokens ||
       !expert_x || !expert_meta)
     return MOE_A2A_EINVAL;
@@ -1471,18 +1590,27 @@ int moe_a2a_dispatch_recv(const moe_a2a_shape* s, const void* recv_buf, const in
   if (!items_fit((long long)g.nle * g.max_recv, g.wchunks)) return MOE_A2A_EINVAL;
   const int grid = g.nle + mover_blocks(group_items(rows_hint, g));
   hipStream_t st = (hipStream_t)stream;
-#define LAUNCH(V, NVW)                                                                      \
-  dispatch_recv_kernel<V, NVW><<<grid, 64 * ROWS, 0, st>>>(                                 \
+  const bool planned = send_back_plan && plan_supported(s);
+#define LAUNCH_P(V, NVW, PLAN)                                                              \
+  dispatch_recv_kernel<V, NVW, PLAN><<<grid, 64 * ROWS, 0, st>>>(                           \
       (const V*)recv_buf, recv_meta, recv_counts, s->world_size, rows_hint, capacity_rows,   \
-      g.nle, g.magic, g.max_recv, g.row_vecs, g.wchunks, expert_num_tokens, (V*)expert_x, expert_meta)
+      g.nle, g.magic, g.max_recv, g.row_vecs, g.wchunks, expert_num_tokens, (V*)expert_x,    \
+      expert_meta, send_back_plan)
+#define LAUNCH(V, NVW)                     \
+  do {                                     \
+    if (planned) LAUNCH_P(V, NVW, true);   \
+    else LAUNCH_P(V, NVW, false);          \
+  } while (0)
   MOE_A2A_FOR_WAVE_KERNEL(g, LAUNCH);
 #undef LAUNCH
+#undef LAUNCH_P
   return launch_status();
 }
 
 int moe_a2a_combine_send(const moe_a2a_shape* s, const void* expert_y, const int32_t* expert_meta,
                          const int32_t* expert_num_tokens, int32_t rows_hint,
-                         int32_t capacity_rows, void* send_buf, int32_t* send_meta, int32_t* send_counts, void* stream) {
+                         int32_t capacity_rows, void* send_buf, int32_t* send_meta, int32_t* send_counts,
+                         const int32_t* send_back_plan, void* stream) {
   if (!shape_ok(s) || rows_hint < 0 || capacity_rows < 0 || !expert_y || !expert_meta ||
       !expert_num_tokens || !send_counts)
     return MOE_A2A_EINVAL;
@@ -1493,14 +1621,17 @@ int moe_a2a_combine_send(const moe_a2a_shape* s, const void* expert_y, const int
   if (!items_fit((long long)g.nle * g.max_recv, g.wchunks)) return MOE_A2A_EINVAL;
   const int grid = s->world_size + mover_blocks(group_items(rows_hint, g));
   hipStream_t st = (hipStream_t)stream;
-#define LAUNCH_S(V, NVW, SMALL)                                                                \
-  combine_send_kernel<V, NVW, SMALL><<<grid, 64 * ROWS, 0, st>>>(                             \
+  const bool planned = send_back_plan && plan_supported(s);
+#define LAUNCH_S(V, NVW, SMALL, PLAN)                                                          \
+  combine_send_kernel<V, NVW, SMALL, PLAN><<<grid, 64 * ROWS, 0, st>>>(                       \
       (const V*)expert_y, expert_meta, expert_num_tokens, g.nle, g.max_recv, s->world_size,    \
-      g.row_vecs, g.wchunks, capacity_rows, (V*)send_buf, send_meta, send_counts)
-#define LAUNCH(V, NVW)                        \
-  do {                                        \
-    if (g.nle <= 64) LAUNCH_S(V, NVW, true);  \
-    else LAUNCH_S(V, NVW, false);             \
+      g.row_vecs, g.wchunks, capacity_rows, (V*)send_buf, send_meta, send_counts,              \
+      send_back_plan)
+#define LAUNCH(V, NVW)                                   \
+  do {                                                   \
+    if (planned) LAUNCH_S(V, NVW, true, true);           \
+    else if (g.nle <= 64) LAUNCH_S(V, NVW, true, false); \
+    else LAUNCH_S(V, NVW, false, false);                 \
   } while (0)
   MOE_A2A_FOR_WAVE_KERNEL(g, LAUNCH);
 #undef LAUNCH

@@ -61,6 +61,8 @@ def parse_args():
                     help="whole steps per graph in the per-kernel (leave-one-out) timing")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="target CPU time of the cpu_baseline sample")
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
+    ap.add_argument("--no-placement-plan", action="store_true",
+                    help="combine_send ranks its rows by scanning instead of using dispatch_recv's plan")
     ap.add_argument("--alone", action="store_true",
                     help="also time every kernel back to back with itself (warm inputs)")
     return ap.parse_args()
@@ -104,7 +106,7 @@ def main():
     data = [d.to(dev) for _, d, _, _ in world]
 
     # ---- set-up: the whole job once, so rank 0's inbound buffers hold the peers' segments
-    lw = LocalWorld(cfg, W, device=dev)
+    lw = LocalWorld(cfg, W, device=dev, reuse_placement=not args.no_placement_plan)
     ys0 = [y.clone() for y in lw.run(data)]
     torch.cuda.synchronize()
     r0 = args.rank

@@ -128,6 +128,14 @@ int moe_a2a_plan_send(const moe_a2a_shape* shape, const int32_t* indices,
  *                       written (the reference leaves the rest uninitialised
  *                       too: torch.empty at reference.py:127)
  *   expert_meta [nle, max_recv, 5] out, same rule
+ *   send_back_plan [2 * num_experts] int32 out, optional (may be NULL):
+ *                       where moe_a2a_combine_send will put every row, worked
+ *                       out here because the keys are being counted anyway.
+ *                       Opaque to the caller. Written only when W <= 64 and
+ *                       nle <= 64 (ignored otherwise, by both entry points).
+ *                       It takes the origin of a row from the segment the row
+ *                       arrived in, which is what every sender writes into
+ *                       meta[1] (all2all/reference.py:84).
  * A row whose position inside its expert would reach max_recv is not stored;
  * expert_num_tokens still counts it, so overflow is visible to the caller.
  */
@@ -135,7 +143,8 @@ int moe_a2a_dispatch_recv(const moe_a2a_shape* shape, const void* recv_buf,
                           const int32_t* recv_meta, const int32_t* recv_counts,
                           int32_t rows_hint, int32_t capacity_rows,
                           int32_t* expert_num_tokens, void* expert_x,
-                          int32_t* expert_meta, void* stream);
+                          int32_t* expert_meta, int32_t* send_back_plan,
+                          void* stream);
 
 /*
  * Combine, send side: expert-major results -> rows grouped by origin rank.
@@ -147,13 +156,20 @@ int moe_a2a_dispatch_recv(const moe_a2a_shape* shape, const void* recv_buf,
  *   send_buf    [R, H] out, send_meta [R, 5] out (meta rows copied unchanged);
  *               capacity_rows is their allocation
  *   send_counts [W] int32 out
+ *   send_back_plan [2 * num_experts] int32, optional (may be NULL): the plan
+ *               moe_a2a_dispatch_recv wrote together with this expert_meta and
+ *               expert_num_tokens. With it rows are placed without reading the
+ *               origin column of expert_meta, so it must be passed only while
+ *               both are as that call left them (the order of the rows of an
+ *               expert, the origin ranks, the counts); pass NULL after changing
+ *               any of them. Results are the same with and without it.
  */
 int moe_a2a_combine_send(const moe_a2a_shape* shape, const void* expert_y,
                          const int32_t* expert_meta,
                          const int32_t* expert_num_tokens, int32_t rows_hint,
                          int32_t capacity_rows, void* send_buf,
                          int32_t* send_meta, int32_t* send_counts,
-                         void* stream);
+                         const int32_t* send_back_plan, void* stream);
 
 /*
  * Combine, receive side: weighted sum back into token order.

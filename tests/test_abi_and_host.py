@@ -64,13 +64,13 @@ def test_bad_arguments_are_rejected_without_touching_the_gpu():
     assert lib.moe_a2a_dispatch_send(C.byref(ok), one, one, 257, one, one, one, None, None) == -1
     assert lib.moe_a2a_dispatch_send(C.byref(ok), None, one, 4, one, one, one, None, None) == -1
     assert lib.moe_a2a_dispatch_send(C.byref(ok), C.c_void_p(17), one, 4, one, one, one, None, None) == -2
-    assert lib.moe_a2a_dispatch_recv(C.byref(ok), one, one, None, 4, 4, one, one, one, None) == -1
-    assert lib.moe_a2a_dispatch_recv(C.byref(ok), one, one, one, 4, -1, one, one, one, None) == -1
-    assert lib.moe_a2a_dispatch_recv(C.byref(ok), one, one, one, 4, 1 << 30, one, one, one, None) == -1
-    assert lib.moe_a2a_dispatch_recv(C.byref(ok), None, one, one, 0, 4, one, one, one, None) == -1
-    assert lib.moe_a2a_combine_send(C.byref(ok), one, one, one, -1, 4, one, one, one, None) == -1
-    assert lib.moe_a2a_combine_send(C.byref(ok), one, one, one, 4, -1, one, one, one, None) == -1
-    assert lib.moe_a2a_combine_send(C.byref(ok), one, one, one, 4, 4, None, one, one, None) == -1
+    assert lib.moe_a2a_dispatch_recv(C.byref(ok), one, one, None, 4, 4, one, one, one, None, None) == -1
+    assert lib.moe_a2a_dispatch_recv(C.byref(ok), one, one, one, 4, -1, one, one, one, None, None) == -1
+    assert lib.moe_a2a_dispatch_recv(C.byref(ok), one, one, one, 4, 1 << 30, one, one, one, None, None) == -1
+    assert lib.moe_a2a_dispatch_recv(C.byref(ok), None, one, one, 0, 4, one, one, one, None, None) == -1
+    assert lib.moe_a2a_combine_send(C.byref(ok), one, one, one, -1, 4, one, one, one, None, None) == -1
+    assert lib.moe_a2a_combine_send(C.byref(ok), one, one, one, 4, -1, one, one, one, None, None) == -1
+    assert lib.moe_a2a_combine_send(C.byref(ok), one, one, one, 4, 4, None, one, one, None, None) == -1
     assert lib.moe_a2a_combine_recv(C.byref(ok), one, one, one, 4, 4, one, 4, one, 0, 7, None) == -1
     assert lib.moe_a2a_combine_recv(C.byref(ok), one, one, one, 4, -1, one, 4, one, 0, 1, None) == -1
     assert lib.moe_a2a_combine_recv(C.byref(ok), one, one, one, 4, 1 << 30, one, 4, one, 0, 1, None) == -1

@@ -57,9 +57,9 @@ def assert_rank_matches(tr_gpu: dict, t: orc.RankTrace, T: int, K: int, tag: str
     assert eq(bits(tr_gpu["y"][:T]), t.y), tag
 
 
-def run_and_compare(world, exact_hints=True, accumulate=False):
+def run_and_compare(world, exact_hints=True, accumulate=False, reuse_placement=True):
     cfg = world[0][0]
-    lw = LocalWorld(cfg, len(world), device=DEV, exact_hints=exact_hints)
+    lw = LocalWorld(cfg, len(world), device=DEV, exact_hints=exact_hints, reuse_placement=reuse_placement)
     dev = to_dev(world)
     ys = lw.run([d for _, d, _, _ in dev], accumulate=accumulate)
     torch.cuda.synchronize()
@@ -433,7 +433,7 @@ def test_counts_beyond_capacity_are_cut_off():
     # ---- dispatch_recv: counts claim 40 rows, the buffers are said to hold 24
     meta_np = np.zeros((ALLOC, 5), np.int32)
     meta_np[:, 0] = rng.integers(0, nle, ALLOC)
-    meta_np[:, 1] = np.repeat(np.arange(W), ALLOC // W)
+    meta_np[:, 1] = np.minimum(np.arange(ALLOC) // 10, W - 1)  # the source of a row is the segment it arrives in
     meta_np[:, 2] = rng.integers(0, max_T, ALLOC)
     meta_np[:, 3] = rng.integers(0, K, ALLOC)
     recv_buf, recv_meta = rows(ALLOC), torch.from_numpy(meta_np).to(DEV)
@@ -444,7 +444,7 @@ def test_counts_beyond_capacity_are_cut_off():
     for hint in (0, 7, CAP, 40, 1000):
         num.fill_(SENT); em.fill_(SENT)
         _lib.call("moe_a2a_dispatch_recv", shape, p(recv_buf), p(recv_meta), p(counts40), hint, CAP,
-                  p(num), p(ex), p(em), st)
+                  p(num), p(ex), p(em), None, st)
         torch.cuda.synchronize()
         cnt, local, pos, order = orc.expert_placement(meta_np[:CAP], nle)
         assert np.array_equal(num.cpu().numpy(), cnt), hint
@@ -469,10 +469,18 @@ def test_counts_beyond_capacity_are_cut_off():
     back_buf = torch.zeros(ALLOC, H, dtype=torch.bfloat16, device=DEV)
     back_meta = torch.full((ALLOC, 5), SENT, dtype=torch.int32, device=DEV)
     back_counts = torch.full((W,), SENT, dtype=torch.int32, device=DEV)
-    for hint in (0, CAP, 40, 1000):
+    # the plan of these 40 rows, as stage 2 writes it next to the same placement
+    plan = torch.full((2 * W * nle,), SENT, dtype=torch.int32, device=DEV)
+    num_b, ex_b, em_b = torch.empty_like(num), torch.empty_like(ex), torch.empty_like(em)
+    _lib.call("moe_a2a_dispatch_recv", shape, p(recv_buf), p(recv_meta), p(counts40), 40, 40,
+              p(num_b), p(ex_b), p(em_b), p(plan), st)
+    torch.cuda.synchronize()
+    assert np.array_equal(num_b.cpu().numpy(), cnt40)
+    assert np.array_equal(valid_rows(em_b, cnt40).numpy(), stream_meta)
+    for hint, use_plan in ((0, None), (CAP, None), (40, None), (1000, None), (0, plan), (40, plan)):
         back_meta.fill_(SENT); back_buf.zero_()
         _lib.call("moe_a2a_combine_send", shape, p(ey), p(em), p(num40), hint, CAP, p(back_buf),
-                  p(back_meta), p(back_counts), st)
+                  p(back_meta), p(back_counts), None if use_plan is None else p(use_plan), st)
         torch.cuda.synchronize()
         bc, bo = orc.return_order(stream_meta, W)
         assert np.array_equal(back_counts.cpu().numpy(), bc), hint   # counts are the true ones
@@ -504,3 +512,35 @@ def test_counts_beyond_capacity_are_cut_off():
         torch.cuda.synchronize()
         want = orc.combine_recv(bits(recv_buf[:CAP]), meta_np[:CAP], weights.cpu().numpy(), max_T, "bf16")
         assert np.array_equal(bits(y), want), hint
+
+
+@pytest.mark.parametrize("name", ["C1", "C2", "C3", "C5"])
+def test_without_placement_plan(name):
+    """Stage 3 ranking its rows by scanning the origin column, as it does for a caller that
+    passes no plan."""
+    run_and_compare(generate_world(WORKLOADS[name], 31), reuse_placement=False)
+
+
+def test_plan_is_set_aside_when_an_expert_overflows():
+    """Every entry of every rank routed to expert 0: more rows than max_recv arrive for it, the
+    surplus is dropped by stage 2 and the plan no longer describes the buffers. Stage 3 must
+    notice and rank by scanning: both settings give the same bits."""
+    spec = dict(world_size=2, num_experts=4, experts_per_token=4, hidden_dim=64, max_num_tokens=6,
+                num_tokens="full", routing="uniform", weights="rand", dtype="bf16")
+    world = generate_world(spec, 11)
+    cfg = world[0][0]
+    outs = []
+    for reuse in (True, False):
+        lw = LocalWorld(cfg, len(world), device=DEV, reuse_placement=reuse)
+        data = [d.to(DEV) for _, d, _, _ in world]
+        for d in data:
+            d.indices = torch.zeros_like(d.indices)
+        ys = lw.run(data)
+        torch.cuda.synchronize()
+        tr = lw.trace[0]
+        assert int(tr["expert_num_tokens"][0]) > lw.ranks[0].max_recv  # the overflow is reported
+        n = int(tr["back_counts"].sum())
+        outs.append([tr["back_counts"].cpu().numpy(), tr["back_meta"][:n].cpu().numpy(), bits(tr["back_buf"][:n])]
+                    + [bits(y) for y in ys])
+    for a, b in zip(*outs):
+        assert np.array_equal(a, b)
