@@ -1502,7 +1502,7 @@ long long group_items(long long rows, const Geometry& g) {
 
 extern "C" {
 
-const char* moe_a2a_version(void) { return "moe_a2a 0.2 gfx950"; }
+const char* moe_a2a_version(void) { return "moe_a2a 0.3 gfx950"; }
 
 const char* moe_a2a_strerror(int status) {
   switch (status) {

@@ -65,7 +65,7 @@ typedef struct moe_a2a_shape {
 } moe_a2a_shape;
 
 /* Library version / build probe. Returns a static string such as
- * "moe_a2a 0.1 gfx950". Never NULL. */
+ * "moe_a2a 0.3 gfx950"; the number changes with the ABI. Never NULL. */
 const char* moe_a2a_version(void);
 
 /* Human-readable text for a status code. Never NULL. */
