@@ -137,6 +137,9 @@ EDGE = {
                                  max_num_tokens=6, num_tokens="full", dtype="bf16"),
     "many_entries_several_key_batches": dict(world_size=2, num_experts=16, experts_per_token=10, hidden_dim=64,
                                              max_num_tokens=300, num_tokens="full", dtype="bf16"),
+    "two_entries_per_token_several_key_batches": dict(world_size=2, num_experts=4, experts_per_token=2,
+                                                      hidden_dim=32, max_num_tokens=2300, num_tokens="full",
+                                                      dtype="fp16"),
     "k_above_fast_list": dict(world_size=2, num_experts=160, experts_per_token=72, hidden_dim=64,
                               max_num_tokens=3, num_tokens="full", dtype="bf16"),
 }
