@@ -263,7 +263,11 @@ class LocalWorld:
         self.ranks = [HIPAllToAll(cfg, r, world_size, device=device, reuse_placement=reuse_placement)
                       for r in range(world_size)]
         self.device = self.ranks[0].device
-        self.exact_hints = exact_hints  # read the counts back to size the copies exactly
+        # True: read the counts back to size every launch exactly (synchronises the host);
+        # False: size for the worst case; "last": reuse what the previous run read back, for
+        # replaying the same job without touching the host (graph capture)
+        self.exact_hints = exact_hints
+        self._last_counts = {}
         self.trace: List[dict] = [dict() for _ in range(world_size)]
 
     def _exchange(self, phase: str, sent: List[Tuple[torch.Tensor, torch.Tensor, torch.Tensor]]):
@@ -271,7 +275,11 @@ class LocalWorld:
         all_counts = torch.stack([s[0] for s in sent])      # [src, dst]
         per_dst = all_counts.t().contiguous()                # [dst, src]
         bound = sent[0][1].shape[0]
-        host = all_counts.cpu().tolist() if self.exact_hints else None
+        if self.exact_hints == "last":  # the counts read back by the previous run of the same job
+            host = self._last_counts[phase]
+        else:
+            host = all_counts.cpu().tolist() if self.exact_hints else None
+            self._last_counts[phase] = host
         got = []
         for r, dst in enumerate(self.ranks):
             rc, rb, rm = dst.inbound_buffers(phase)
