@@ -41,6 +41,15 @@ def test_argument_counts_match_the_header():
         assert n == len(args), (name, n, len(args))
 
 
+def test_integration_notes_bind_the_current_argument_lists():
+    """The ctypes stub printed in INTEGRATION.md must list as many arguments as the header."""
+    text = (ROOT / "INTEGRATION.md").read_text()
+    found = dict(re.findall(r"lib\.(moe_a2a_\w+)\.argtypes\s*=\s*\[(.*?)\]", text))
+    assert found, "no argtypes lines found"
+    for name, args in found.items():
+        assert len([a for a in args.split(",") if a.strip()]) == len(_lib.SIGNATURES[name]), name
+
+
 def test_shape_struct_layout_matches_header():
     fields = re.search(r"typedef struct moe_a2a_shape \{(.*?)\} moe_a2a_shape;", HEADER, flags=re.S).group(1)
     names = re.findall(r"int32_t\s+(\w+);", fields)
