@@ -547,3 +547,16 @@ def test_plan_is_set_aside_when_an_expert_overflows():
                     + [bits(y) for y in ys])
     for a, b in zip(*outs):
         assert np.array_equal(a, b)
+
+
+@pytest.mark.parametrize("inp,out", [("bf16", "fp16"), ("fp16", "bf16")])
+def test_different_input_and_output_types(inp, out):
+    """Tokens travel in `in_dtype`, the expert converts to `out_dtype` (all2all/reference.py:262),
+    the combine runs in `out_dtype`."""
+    spec = dict(world_size=4, num_experts=16, experts_per_token=3, hidden_dim=264, max_num_tokens=20,
+                num_tokens="uniform", routing="uniform", weights="softmax", dtype=inp)
+    world = generate_world(spec, 123)
+    cfg = world[0][0]
+    mixed = MoEConfig(cfg.num_experts, cfg.experts_per_token, cfg.hidden_dim, cfg.max_num_tokens,
+                      in_dtype=DTYPES[inp], out_dtype=DTYPES[out])
+    run_and_compare([(mixed, d, r, w) for (_, d, r, w) in world])
