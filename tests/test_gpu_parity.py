@@ -560,3 +560,20 @@ def test_different_input_and_output_types(inp, out):
     mixed = MoEConfig(cfg.num_experts, cfg.experts_per_token, cfg.hidden_dim, cfg.max_num_tokens,
                       in_dtype=DTYPES[inp], out_dtype=DTYPES[out])
     run_and_compare([(mixed, d, r, w) for (_, d, r, w) in world])
+
+
+def test_repeated_expert_ids_inside_a_token():
+    """The reference draws distinct ids per token, but its loops are defined for any ids
+    (all2all/reference.py:76-86): entries of a token that name the same expert keep their k
+    order everywhere. Ids drawn with replacement, a few tokens with all entries equal."""
+    spec = dict(world_size=4, num_experts=32, experts_per_token=6, hidden_dim=136, max_num_tokens=24,
+                num_tokens="full", routing="uniform", weights="rand", dtype="bf16")
+    world = generate_world(spec, 99)
+    rng = np.random.default_rng(5)
+    for _, d, r, _ in world:
+        ids = rng.integers(0, 32, tuple(d.indices.shape)).astype(np.int32)
+        ids[r] = 7          # one token per rank sends every entry to the same expert
+        ids[r + 4, :3] = 31
+        d.indices = torch.from_numpy(ids)
+    for plan in (True, False):
+        run_and_compare(world, reuse_placement=plan)
