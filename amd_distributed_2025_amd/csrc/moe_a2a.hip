@@ -158,16 +158,17 @@ __device__ __forceinline__ int floormod(int e, int d, uint32_t magic) {
 }
 
 // Inclusive [lo, hi] range of expert ids owned by the same destination as `e`.
-// Ids below 0 and ids >= E form two extra classes before / after all ranks, so
-// the classes always partition the integers and slots stay a permutation.
-__device__ __forceinline__ void dest_class(int e, int nle, int E, uint32_t magic, int& lo, int& hi,
-                                           int& d) {
-  if (e < 0) {
-    lo = INT_MIN; hi = -1; d = -1;
-  } else if (e >= E) {
-    lo = E; hi = INT_MAX; d = INT_MAX;
+// Ids outside [0, E) name no destination: they form one class after all ranks
+// (compared as unsigned numbers, a negative id is just a large one), so the
+// classes still partition the integers, slots stay a permutation, the rows of
+// the real destinations sit where the counts say, and the stray rows end up
+// behind them, where no exchange looks.
+__device__ __forceinline__ void dest_class(int e, int nle, int E, uint32_t magic, uint32_t& lo,
+                                           uint32_t& hi) {
+  if ((uint32_t)e >= (uint32_t)E) {
+    lo = (uint32_t)E; hi = UINT_MAX;
   } else {
-    d = (nle == 1) ? e : (int)__umulhi((uint32_t)e, magic);
+    const uint32_t d = (nle == 1) ? (uint32_t)e : __umulhi((uint32_t)e, magic);
     lo = d * nle; hi = lo + nle - 1;
   }
 }
@@ -382,16 +383,17 @@ __global__ __launch_bounds__(64 * ROWS) void dispatch_send_kernel(
     WavePayload<V, NVW> p;
     p.load(x + (size_t)t * row_vecs, base, row_vecs, lane);
 
-    int rlo[ROWS], rhi[ROWS], e = 0;
+    uint32_t rlo[ROWS], rhi[ROWS];
+    int e = 0;
 #pragma unroll
     for (int r = 0; r < ROWS; ++r) {
-      int d;
-      dest_class(re[r], nle, E, magic, rlo[r], rhi[r], d);
+      dest_class(re[r], nle, E, magic, rlo[r], rhi[r]);
       if (r == wave) e = re[r];
     }
     int cnt[ROWS];
     scan.finish(key, S, [&](int r, int e2, int i2) {
-      return (e2 < rlo[r]) | ((e2 <= rhi[r]) & (e2 >= rlo[r]) & (i2 < i0 + r));
+      const uint32_t u2 = (uint32_t)e2;
+      return (u2 < rlo[r]) | ((u2 <= rhi[r]) & (u2 >= rlo[r]) & (i2 < i0 + r));
     }, cnt);
     const int slot = rows_reduce(cnt, part, parity, wave, lane);
 
@@ -413,8 +415,8 @@ __global__ __launch_bounds__(64 * ROWS) void dispatch_send_kernel(
 // keys, and the row held in registers is stored to each of their slots. Compared
 // with a wave per entry this reads every source row once instead of K times and
 // issues an eighth of the key loads. The order is carried by one composite key
-// per entry, class * S + i with class = 0 (id < 0), 1 + destination, W + 1
-// (id >= E): entry a precedes entry b exactly when its composite key is smaller.
+// per entry, class * S + i with class = destination, or W for an id outside
+// [0, E): entry a precedes entry b exactly when its composite key is smaller.
 // The host uses this kernel when (W + 2) * S fits an int.
 
 constexpr int FAN = 8;
@@ -427,12 +429,13 @@ __global__ __launch_bounds__(BLOCK) void dispatch_fanout_kernel(
   __shared__ int part[2 * NWAVES * FAN];
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const int S = T * K;
+  // destination rank, or W for an id outside [0, E)
   auto klass = [&](int e) {
-    return e < 0 ? 0 : e >= E ? W + 1 : 1 + (nle == 1 ? e : (int)__umulhi((uint32_t)e, magic));
+    return (uint32_t)e >= (uint32_t)E ? W : nle == 1 ? e : (int)__umulhi((uint32_t)e, magic);
   };
 
   if ((int)blockIdx.x < W) {
-    const int want = blockIdx.x + 1;
+    const int want = blockIdx.x;
     int c = count_keys<BLOCK>(S, StridedKeys{indices, 1}, [&](int e, int) { return klass(e) == want; });
     c = block_sum<NWAVES>(c, part);
     if (tid == 0) send_counts[blockIdx.x] = c;

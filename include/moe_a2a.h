@@ -86,6 +86,10 @@ const char* moe_a2a_strerror(int status);
  *   send_counts [W] int32        out: rows per destination rank
  *   send_slot   [num_tokens*K]   out, optional (may be NULL): row of
  *                                send_buf that entry t*K+k went to
+ * An entry whose expert id is outside [0, E) names no destination (the
+ * reference indexes out of range there, all2all/reference.py:80-81): its row is
+ * placed behind the rows of all destinations, in (t, k) order, and counted for
+ * no rank, so it is never exchanged and adds nothing to the combine.
  */
 int moe_a2a_dispatch_send(const moe_a2a_shape* shape, const void* x,
                           const int32_t* indices, int32_t num_tokens,

@@ -577,3 +577,46 @@ def test_repeated_expert_ids_inside_a_token():
         d.indices = torch.from_numpy(ids)
     for plan in (True, False):
         run_and_compare(world, reuse_placement=plan)
+
+
+@pytest.mark.parametrize("K", [2, 6])
+def test_expert_ids_outside_the_range_are_set_aside(K):
+    """Ids below 0 or at/above E name no destination. Their rows must land behind all
+    destinations' rows without disturbing them, and the result must equal the oracle's on a job
+    where those entries point at a real expert with weight 0 (an addend of +0 changes nothing)."""
+    from amd_distributed_2025_amd import HIPAllToAll
+
+    E, W = 16, 4
+    spec = dict(world_size=W, num_experts=E, experts_per_token=K, hidden_dim=72, max_num_tokens=18,
+                num_tokens="full", routing="uniform", weights="rand", dtype="bf16")
+    world = generate_world(spec, 17)
+    rng = np.random.default_rng(8)
+    substitute = [(c, d.to("cpu"), r, w) for (c, d, r, w) in world]   # separate tensors
+    for (_, d, r, _), (_, ds, _, _) in zip(world, substitute):
+        ids = d.indices.numpy().copy()
+        stray = rng.random(ids.shape) < 0.2
+        stray[0, 0] = True
+        bad = np.where(rng.random(ids.shape) < 0.5, -1 - rng.integers(0, 5, ids.shape), E + rng.integers(0, 5, ids.shape))
+        d.indices = torch.from_numpy(np.where(stray, bad, ids).astype(np.int32))
+        ds.indices = torch.from_numpy(ids.astype(np.int32))
+        ds.weights = torch.from_numpy(np.where(stray, np.float32(0), d.weights.numpy()).astype(np.float32))
+        ds.x = d.x
+    want = run_oracle(substitute)
+    cfg = world[0][0]
+    lw = LocalWorld(cfg, W, device=DEV)
+    ys = lw.run([d.to(DEV) for _, d, _, _ in world])
+    torch.cuda.synchronize()
+    nle = E // W
+    for r in range(W):
+        assert np.array_equal(bits(ys[r]), want[r].y), r
+        ids = world[r][1].indices.numpy().ravel()
+        ok = (ids >= 0) & (ids < E)
+        counts = lw.trace[r]["send_counts"].cpu().numpy()
+        assert np.array_equal(counts, np.bincount(ids[ok] // nle, minlength=W)), r
+        n = int(counts.sum())
+        meta = lw.trace[r]["send_meta"].cpu().numpy()
+        sent = meta[:n]
+        assert ((sent[:, 0] >= 0) & (sent[:, 0] < E)).all() and (np.diff(sent[:, 0] // nle) >= 0).all(), r
+        behind = meta[n: ids.size]
+        assert np.array_equal(behind[:, 0], ids[~ok]), r                      # in (t, k) order
+        assert np.array_equal(behind[:, 2] * K + behind[:, 3], np.flatnonzero(~ok)), r
