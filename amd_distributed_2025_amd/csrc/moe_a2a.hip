@@ -1034,8 +1034,10 @@ __global__ __launch_bounds__(64 * ROWS) void combine_send_kernel(
     p.load(expert_y + row * row_vecs, base, row_vecs, lane);
 
     int cnt[ROWS];
+    // origins compared as unsigned numbers: a row whose meta names no rank (negative, or W and
+    // above) sorts behind the rows of every real origin instead of shifting their segments
     scan.finish(key, R, [&](int r, int d2, int g2) {
-      return (d2 < rd[r]) | ((d2 == rd[r]) & (g2 < g0 + r));
+      return ((uint32_t)d2 < (uint32_t)rd[r]) | ((d2 == rd[r]) & (g2 < g0 + r));
     }, cnt);
     const int slot = rows_reduce(cnt, part, parity, wave, lane);
 

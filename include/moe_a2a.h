@@ -160,6 +160,8 @@ int moe_a2a_dispatch_recv(const moe_a2a_shape* shape, const void* recv_buf,
  *   send_buf    [R, H] out, send_meta [R, 5] out (meta rows copied unchanged);
  *               capacity_rows is their allocation
  *   send_counts [W] int32 out
+ *               A row whose meta[1] names no rank (below 0, W or above) is
+ *               counted for nobody and placed behind the rows of all origins.
  *   send_back_plan [2 * num_experts] int32, optional (may be NULL): the plan
  *               moe_a2a_dispatch_recv wrote together with this expert_meta and
  *               expert_num_tokens. With it rows are placed without reading the

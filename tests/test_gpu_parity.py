@@ -620,3 +620,47 @@ def test_expert_ids_outside_the_range_are_set_aside(K):
         behind = meta[n: ids.size]
         assert np.array_equal(behind[:, 0], ids[~ok]), r                      # in (t, k) order
         assert np.array_equal(behind[:, 2] * K + behind[:, 3], np.flatnonzero(~ok)), r
+
+
+def test_send_back_rows_whose_meta_names_no_rank_go_last():
+    """Stage 3 ranking by the origin column (no plan): origins outside [0, W) must not shift the
+    segments of the real origins; such rows are counted for nobody and placed behind."""
+    import ctypes as C
+    from amd_distributed_2025_amd import HIPAllToAll, _lib
+
+    W, nle, K, H, max_T = 4, 2, 2, 40, 4
+    cfg = MoEConfig(W * nle, K, H, max_T, in_dtype=torch.bfloat16, out_dtype=torch.bfloat16)
+    a = HIPAllToAll(cfg, 1, W, device=DEV)
+    max_recv = max_T * W
+    counts = np.array([5, 7], np.int32)
+    origin = [np.array([0, 0, -3, 2, 3]), np.array([0, 1, 1, 9, 2, -1, 3])]
+    rng = np.random.default_rng(2)
+    ey = torch.zeros(nle, max_recv, H, dtype=torch.bfloat16, device=DEV)
+    em = torch.full((nle, max_recv, 5), -7, dtype=torch.int32, device=DEV)
+    stream_meta, stream_rows = [], []
+    for le in range(nle):
+        n = int(counts[le])
+        m = np.zeros((n, 5), np.int32)
+        m[:, 0] = 2 + le; m[:, 1] = origin[le]; m[:, 2] = rng.integers(0, max_T, n); m[:, 3] = rng.integers(0, K, n)
+        rows = torch.from_numpy(rng.integers(0, 0x4400, (n, H), dtype=np.int16)).view(torch.bfloat16)
+        ey[le, :n] = rows.to(DEV); em[le, :n] = torch.from_numpy(m).to(DEV)
+        stream_meta.append(m); stream_rows.append(bits(rows))
+    stream_meta, stream_rows = np.concatenate(stream_meta), np.concatenate(stream_rows)
+    real = (stream_meta[:, 1] >= 0) & (stream_meta[:, 1] < W)
+    want_counts, order = orc.return_order(stream_meta[real], W)
+    n_real, n_all = int(real.sum()), int(counts.sum())
+    back_buf = torch.zeros(n_all, H, dtype=torch.bfloat16, device=DEV)
+    back_meta = torch.zeros(n_all, 5, dtype=torch.int32, device=DEV)
+    back_counts = torch.zeros(W, dtype=torch.int32, device=DEV)
+    p = lambda t: C.c_void_p(t.data_ptr())
+    _lib.call("moe_a2a_combine_send", C.byref(a.shape), p(ey), p(em), p(torch.from_numpy(counts).to(DEV)),
+              n_all, n_all, p(back_buf), p(back_meta), p(back_counts), None,
+              C.c_void_p(torch.cuda.current_stream().cuda_stream))
+    torch.cuda.synchronize()
+    assert np.array_equal(back_counts.cpu().numpy(), want_counts)
+    assert np.array_equal(back_meta.cpu().numpy()[:n_real], stream_meta[real][order])
+    assert np.array_equal(bits(back_buf[:n_real]), stream_rows[real][order])
+    # the strays follow, ordered by their origin read as an unsigned number, then by stream position
+    stray = np.flatnonzero(~real)
+    stray = stray[np.argsort(stream_meta[stray, 1].astype(np.uint32), kind="stable")]
+    assert np.array_equal(back_meta.cpu().numpy()[n_real:], stream_meta[stray])
