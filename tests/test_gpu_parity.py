@@ -125,6 +125,10 @@ def test_reference_test_shapes_fp16(i):
 EDGE = {
     "odd_hidden_2byte_path": dict(world_size=4, num_experts=8, experts_per_token=2, hidden_dim=100,
                                   max_num_tokens=9, num_tokens="uniform", dtype="bf16"),
+    "hidden_dim_odd": dict(world_size=2, num_experts=4, experts_per_token=2, hidden_dim=37,
+                           max_num_tokens=5, num_tokens="full", dtype="fp16"),
+    "hidden_dim_one": dict(world_size=2, num_experts=6, experts_per_token=3, hidden_dim=1,
+                           max_num_tokens=7, num_tokens="full", dtype="bf16"),
     "hidden_16B_not_vec_multiple": dict(world_size=2, num_experts=4, experts_per_token=2, hidden_dim=2056,
                                         max_num_tokens=5, num_tokens="full", dtype="fp16"),
     "single_token_single_k": dict(world_size=8, num_experts=8, experts_per_token=1, hidden_dim=64,
