@@ -144,6 +144,9 @@ EDGE = {
     "two_entries_per_token_several_key_batches": dict(world_size=2, num_experts=4, experts_per_token=2,
                                                       hidden_dim=32, max_num_tokens=2300, num_tokens="full",
                                                       dtype="fp16"),
+    "many_tokens_sixteen_key_batches": dict(world_size=4, num_experts=32, experts_per_token=8, hidden_dim=264,
+                                            max_num_tokens=2048, num_tokens="uniform", routing="zipf",
+                                            dtype="bf16"),
     "k_above_fast_list": dict(world_size=2, num_experts=160, experts_per_token=72, hidden_dim=64,
                               max_num_tokens=3, num_tokens="full", dtype="bf16"),
 }
