@@ -42,7 +42,7 @@ def test_argument_counts_match_the_header():
 
 
 def test_integration_notes_bind_the_current_argument_lists():
-    """The ctypes stub printed in INTEGRATION.md must list as many arguments as the header."""
+    """The ctypes stub printed in the integration notes must list as many arguments as the header."""
     text = (ROOT / "INTEGRATION.md").read_text()
     found = dict(re.findall(r"lib\.(moe_a2a_\w+)\.argtypes\s*=\s*\[(.*?)\]", text))
     assert found, "no argtypes lines found"
