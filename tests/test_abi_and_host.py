@@ -50,6 +50,24 @@ def test_integration_notes_bind_the_current_argument_lists():
         assert len([a for a in args.split(",") if a.strip()]) == len(_lib.SIGNATURES[name]), name
 
 
+@pytest.mark.parametrize("compiler,std,suffix", [("gcc", "-std=c99", ".c"), ("g++", "-std=c++11", ".cpp")])
+def test_header_is_plain_c_and_cxx(tmp_path, compiler, std, suffix):
+    """A C or C++ caller needs nothing but the header: it must compile on its own, pedantically,
+    and every declared entry point must be usable as a function pointer."""
+    import shutil
+    import subprocess
+
+    if shutil.which(compiler) is None:
+        pytest.skip(f"{compiler} not installed")
+    src = tmp_path / ("use_header" + suffix)
+    uses = "\n".join(f"  (void)&{name};" for name in declared_functions())
+    src.write_text('#include "moe_a2a.h"\nint main(void) {\n  moe_a2a_shape s = {8, 0, 256, 8, 7168, 256};\n'
+                   "  (void)s;\n" + uses + "\n  return MOE_A2A_OK;\n}\n")
+    r = subprocess.run([compiler, std, "-Wall", "-Wextra", "-Werror", "-pedantic", "-fsyntax-only",
+                        f"-I{ROOT / 'include'}", str(src)], capture_output=True, text=True)
+    assert r.returncode == 0, r.stderr
+
+
 def test_shape_struct_layout_matches_header():
     fields = re.search(r"typedef struct moe_a2a_shape \{(.*?)\} moe_a2a_shape;", HEADER, flags=re.S).group(1)
     names = re.findall(r"int32_t\s+(\w+);", fields)
