@@ -514,6 +514,125 @@ __global__ __launch_bounds__(BLOCK) void dispatch_fanout_kernel(
   }
 }
 
+// The same fan-out for rows longer than 256 vectors: a workgroup of BLK = 512
+// lanes holds one vector per lane, so a row is cut into half as many chunks and
+// its K entries are ranked half as often. A lane compares 2048 / BLK keys per
+// batch; the per-wave counts travel as 16-bit pairs (entry g with entry g + 4),
+// are summed across the waves by the DPP row scan of one wave (a row of 16
+// lanes per pair) and come back through LDS. Needs S < 65536 for the pairs not
+// to carry into each other (a slot is below S). Measured at K = 8, H = 7168:
+// the whole step 0.3 us shorter than with 256 lanes; 1024 lanes (one chunk per
+// row) 0.5 us longer.
+
+template <typename V, int BLK>
+__global__ __launch_bounds__(BLK) void dispatch_fanout_wide_kernel(
+    const V* __restrict__ x, const int* __restrict__ indices, int T, int K, int nle, int E, int W,
+    uint32_t magic, int rank, int row_vecs, int chunks, V* __restrict__ send_buf,
+    int* __restrict__ send_meta, int* __restrict__ send_counts, int* __restrict__ send_slot) {
+  constexpr int NW = BLK / 64;
+  constexpr int KEYS = SCAN_UNROLL * BLOCK / BLK;  // a batch stays SCAN_UNROLL * BLOCK keys
+  constexpr int PAIRS = FAN / 2;
+  static_assert(NW <= 16 && KEYS >= 1, "one DPP row of 16 lanes sums the waves");
+  __shared__ int part[NW * PAIRS];
+  __shared__ int total[PAIRS];
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int S = T * K;
+  // destination rank, or W for an id outside [0, E)
+  auto klass = [&](int e) {
+    return (uint32_t)e >= (uint32_t)E ? W : nle == 1 ? e : (int)__umulhi((uint32_t)e, magic);
+  };
+
+  if ((int)blockIdx.x < W) {
+    const int want = blockIdx.x;
+    int c = count_keys<BLK>(S, StridedKeys{indices, 1}, [&](int e, int) { return klass(e) == want; });
+    c = block_sum<NW>(c, part);
+    if (tid == 0) send_counts[blockIdx.x] = c;
+    return;
+  }
+
+  const int items = T * chunks, movers = gridDim.x - W;
+  for (int q = blockIdx.x - W; q < items; q += movers) {
+    const int t = chunks == 1 ? q : q / chunks, c = q - t * chunks;
+    const int col = c * BLK + tid;
+    const int i0 = t * K;
+
+    int key[KEYS];
+#pragma unroll
+    for (int u = 0; u < KEYS; ++u) key[u] = indices[min(tid + u * BLK, S - 1)];
+    const V v = stream_load(x + (size_t)t * row_vecs + min(col, row_vecs - 1));
+
+    for (int g0 = 0; g0 < K; g0 += FAN) {
+      int mine[FAN];
+#pragma unroll
+      for (int g = 0; g < FAN; ++g) {
+        const int i = i0 + min(g0 + g, K - 1);
+        mine[g] = klass(indices[i]) * S + i;
+      }
+      int cnt[FAN];
+#pragma unroll
+      for (int g = 0; g < FAN; ++g) cnt[g] = 0;
+      auto consume = [&](const int (&k)[KEYS], int b) {
+#pragma unroll
+        for (int u = 0; u < KEYS; ++u) {
+          const int i2 = b + tid + u * BLK;
+          const int ck = i2 < S ? klass(k[u]) * S + i2 : INT_MAX;
+#pragma unroll
+          for (int g = 0; g < FAN; ++g) cnt[g] += (int)(ck < mine[g]);
+        }
+      };
+      consume(key, 0);
+      for (int b = KEYS * BLK; b < S; b += KEYS * BLK) {
+        int more[KEYS];
+#pragma unroll
+        for (int u = 0; u < KEYS; ++u) more[u] = indices[min(b + tid + u * BLK, S - 1)];
+        consume(more, b);
+      }
+
+#pragma unroll
+      for (int h = 0; h < PAIRS; ++h) {
+        const int sum = wave_sum(cnt[h] | (cnt[h + PAIRS] << 16));
+        if (lane == 0) part[wave * PAIRS + h] = sum;
+      }
+      lds_barrier();
+      if (wave == 0) {  // row h of 16 lanes adds up pair h of every wave
+        const int h = lane >> 4, w = lane & 15;
+        int sum = w < NW ? part[w * PAIRS + h] : 0;
+        sum = dpp_add<0x111, 0xf>(sum);
+        sum = dpp_add<0x112, 0xf>(sum);
+        sum = dpp_add<0x114, 0xf>(sum);
+        sum = dpp_add<0x118, 0xf>(sum);
+        if (w == 15) total[h] = sum;
+      }
+      lds_barrier();
+      // no third barrier: `part` is next written before a barrier that wave 0 only reaches after
+      // it has read `part`, and `total` after a barrier every wave reaches after reading it
+      int slot[FAN];
+#pragma unroll
+      for (int h = 0; h < PAIRS; ++h) {
+        const int both = total[h];
+        slot[h] = both & 0xffff;
+        slot[h + PAIRS] = (int)((unsigned)both >> 16);
+      }
+      const int live = min(FAN, K - g0);
+#pragma unroll
+      for (int g = 0; g < FAN; ++g) {
+        if (g < live && col < row_vecs)
+          row_store<(MOE_A2A_NT_SEND != 0)>(send_buf + (size_t)slot[g] * row_vecs + col, v);
+      }
+      if (c == 0 && tid < live * META) {
+        const int g = tid / META, f = tid - g * META;
+        int mine_slot = 0;
+#pragma unroll
+        for (int gg = 0; gg < FAN; ++gg) mine_slot = gg == g ? slot[gg] : mine_slot;
+        const int i = i0 + g0 + g;
+        const int m = f == 0 ? indices[i] : f == 1 ? rank : f == 2 ? t : f == 3 ? g0 + g : 0;
+        send_meta[(size_t)mine_slot * META + f] = m;
+        if (f == 0 && send_slot) send_slot[i] = mine_slot;
+      }
+    }
+  }
+}
+
 // ---------------------------------------------------------------- send plan (counts, offsets, maps)
 //
 // The stable counting sort of stage 1 made explicit, for callers that want the
@@ -1542,6 +1661,23 @@ int moe_a2a_dispatch_send(const moe_a2a_shape* s, const void* x, const int32_t* 
   f.chunks = (f.row_vecs + BLOCK - 1) / BLOCK;
   if (s->experts_per_token >= MOE_A2A_FANOUT_MIN_K && (s->world_size + 2ll) * S <= INT_MAX &&
       items_fit(num_tokens, f.chunks)) {
+#ifndef MOE_A2A_FANOUT_WIDE
+#define MOE_A2A_FANOUT_WIDE 1
+#endif
+    constexpr int WIDE = 2 * BLOCK;  // rows of more than one 256-lane chunk: 512-lane workgroups
+    if (MOE_A2A_FANOUT_WIDE && f.row_vecs > BLOCK && S < 65536) {
+      const int wchunks = (f.row_vecs + WIDE - 1) / WIDE;
+      const int wgrid = s->world_size + mover_blocks((long long)num_tokens * wchunks);
+#define LAUNCH_W(V)                                                                            \
+  dispatch_fanout_wide_kernel<V, WIDE><<<wgrid, WIDE, 0, st>>>(                                \
+      (const V*)x, indices, num_tokens, s->experts_per_token, g.nle, s->num_experts,           \
+      s->world_size, g.magic, s->rank, f.row_vecs, wchunks, (V*)send_buf, send_meta,           \
+      send_counts, send_slot)
+      if (f.vec16) LAUNCH_W(b128);
+      else LAUNCH_W(uint16_t);
+#undef LAUNCH_W
+      return launch_status();
+    }
     const int fgrid = s->world_size + mover_blocks((long long)num_tokens * f.chunks);
 #define LAUNCH(V, NV)                                                                          \
   dispatch_fanout_kernel<V, NV><<<fgrid, BLOCK, 0, st>>>(                                      \
