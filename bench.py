@@ -42,8 +42,8 @@ META_BYTES = 20
 # WRITE_SIZE scaled by what the same counters read for the exchange copy of known size
 # (profiles/c4_rank0_hbm_traffic.md). Other workloads have no committed counter run: traffic is null.
 MEASURED_TRAFFIC_BYTES = {
-    ("C4", 2025, 0): {"dispatch_send": 33.16e6, "dispatch_recv": 57.84e6,
-                   "combine_send": 57.42e6, "combine_recv": 33.00e6},
+    ("C4", 2025, 0): {"dispatch_send": 33.15e6, "dispatch_recv": 57.84e6,
+                   "combine_send": 57.60e6, "combine_recv": 33.00e6},
 }
 
 
