@@ -147,6 +147,12 @@ EDGE = {
     "many_tokens_sixteen_key_batches": dict(world_size=4, num_experts=32, experts_per_token=8, hidden_dim=264,
                                             max_num_tokens=2048, num_tokens="uniform", routing="zipf",
                                             dtype="bf16"),
+    "wide_fanout_several_key_batches": dict(world_size=2, num_experts=8, experts_per_token=8, hidden_dim=2056,
+                                            max_num_tokens=300, num_tokens="full", dtype="bf16"),
+    "wide_fanout_two_byte_rows": dict(world_size=2, num_experts=4, experts_per_token=4, hidden_dim=1001,
+                                      max_num_tokens=6, num_tokens="full", dtype="fp16"),
+    "wide_fanout_twelve_entries": dict(world_size=2, num_experts=24, experts_per_token=12, hidden_dim=4104,
+                                       max_num_tokens=9, num_tokens="uniform", dtype="bf16"),
     "k_above_fast_list": dict(world_size=2, num_experts=160, experts_per_token=72, hidden_dim=64,
                               max_num_tokens=3, num_tokens="full", dtype="bf16"),
 }
