@@ -1679,12 +1679,13 @@ int moe_a2a_dispatch_send(const moe_a2a_shape* s, const void* x, const int32_t* 
       return launch_status();
     }
     const int fgrid = s->world_size + mover_blocks((long long)num_tokens * f.chunks);
-#define LAUNCH(V, NV)                                                                          \
-  dispatch_fanout_kernel<V, NV><<<fgrid, BLOCK, 0, st>>>(                                      \
+#define LAUNCH(V)                                                                              \
+  dispatch_fanout_kernel<V, 1><<<fgrid, BLOCK, 0, st>>>(                                       \
       (const V*)x, indices, num_tokens, s->experts_per_token, g.nle, s->num_experts,           \
       s->world_size, g.magic, s->rank, f.row_vecs, f.chunks, (V*)send_buf, send_meta,          \
       send_counts, send_slot)
-    MOE_A2A_FOR_ROW_KERNEL(f, LAUNCH);
+    if (f.vec16) LAUNCH(b128);  // one vector per lane is the only shape this kernel is launched with
+    else LAUNCH(uint16_t);
 #undef LAUNCH
     return launch_status();
   }
