@@ -1483,6 +1483,41 @@ __global__ __launch_bounds__(BLOCK) void expert_scale_kernel(
   }
 }
 
+// The same for at most 64 local experts and 16-byte vectors: a wave per (row,
+// chunk of 64 * NVW vectors), the expert prefix in one register per lane, the
+// row found with one ballot. No LDS table, no barrier.
+template <int NVW, int DIN, int DOUT>
+__global__ __launch_bounds__(64 * ROWS) void expert_scale_wave_kernel(
+    const b128* __restrict__ expert_x, const int* __restrict__ expert_num_tokens, int nle,
+    int max_recv, float scale, int row_vecs, int chunks, b128* __restrict__ expert_y) {
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const WaveExpertPrefix wp(expert_num_tokens, nle, max_recv);
+  const int items = wp.total * chunks, waves = gridDim.x * ROWS;
+  for (int q = blockIdx.x * ROWS + wave; q < items; q += waves) {
+    const int g = chunks == 1 ? q : q / chunks, c = q - g * chunks;
+    const int base = c * (64 * NVW);
+    int le, first;
+    wp.locate(g, le, first);
+    const size_t row = (size_t)le * max_recv + (g - first);
+    WavePayload<b128, NVW> p;
+    p.load(expert_x + row * row_vecs, base, row_vecs, lane);
+#pragma unroll
+    for (int j = 0; j < NVW; ++j) {
+      uint32_t h[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const uint32_t w = p.v[j][e];
+        // .to(out_dtype), then times (1 + rank) in float32, rounded once
+        const uint32_t o = Pair16<DOUT>::round(Pair16<DIN>::lo(w), Pair16<DIN>::hi(w));
+        h[e] = Pair16<DOUT>::canonical(Pair16<DOUT>::round(__fmul_rn(Pair16<DOUT>::lo(o), scale),
+                                                           __fmul_rn(Pair16<DOUT>::hi(o), scale)));
+      }
+      p.v[j] = from_words<b128>(h);
+    }
+    p.template store<(MOE_A2A_NT_STANDIN != 0)>(expert_y + row * row_vecs, base, row_vecs, lane);
+  }
+}
+
 // ---------------------------------------------------------------- exchange stand-in
 
 template <typename V, int NV>
@@ -1852,9 +1887,39 @@ int moe_a2a_expert_scale(const moe_a2a_shape* s, const void* expert_x,
   const Geometry g = geometry(s, expert_x, expert_y);
   if (g.nle > MAX_LOCAL_EXPERTS) return MOE_A2A_EINVAL;
   if (!items_fit((long long)g.nle * g.max_recv, g.chunks)) return MOE_A2A_EINVAL;
-  const int grid = mover_blocks((long long)rows_hint * g.chunks);
   hipStream_t st = (hipStream_t)stream;
   const float scale = (float)(1 + s->rank);
+#ifndef MOE_A2A_SCALE_WAVES
+#define MOE_A2A_SCALE_WAVES 1
+#endif
+  if (MOE_A2A_SCALE_WAVES && g.vec16 && g.nle <= 64) {
+    const int nvw = g.nvw < 4 ? g.nvw : 4;  // 1, 2 or 4 vectors per lane
+    const int wchunks = (g.row_vecs + 64 * nvw - 1) / (64 * nvw);
+    if (!items_fit((long long)g.nle * g.max_recv, wchunks)) return MOE_A2A_EINVAL;
+    const int wgrid = mover_blocks(((long long)rows_hint * wchunks + ROWS - 1) / ROWS);
+#define LAUNCH_WT(NVW, DI, DO)                                                                 \
+  expert_scale_wave_kernel<NVW, DI, DO><<<wgrid, 64 * ROWS, 0, st>>>(                          \
+      (const b128*)expert_x, expert_num_tokens, g.nle, g.max_recv, scale, g.row_vecs, wchunks,  \
+      (b128*)expert_y)
+#define LAUNCH_W(NVW)                                                                          \
+  do {                                                                                         \
+    if (in_dtype == MOE_A2A_BF16 && out_dtype == MOE_A2A_BF16)                                 \
+      LAUNCH_WT(NVW, MOE_A2A_BF16, MOE_A2A_BF16);                                              \
+    else if (in_dtype == MOE_A2A_F16 && out_dtype == MOE_A2A_F16)                              \
+      LAUNCH_WT(NVW, MOE_A2A_F16, MOE_A2A_F16);                                                \
+    else if (in_dtype == MOE_A2A_F16)                                                          \
+      LAUNCH_WT(NVW, MOE_A2A_F16, MOE_A2A_BF16);                                               \
+    else                                                                                       \
+      LAUNCH_WT(NVW, MOE_A2A_BF16, MOE_A2A_F16);                                               \
+  } while (0)
+    if (nvw == 1) LAUNCH_W(1);
+    else if (nvw == 2) LAUNCH_W(2);
+    else LAUNCH_W(4);
+#undef LAUNCH_W
+#undef LAUNCH_WT
+    return launch_status();
+  }
+  const int grid = mover_blocks((long long)rows_hint * g.chunks);
 #define LAUNCH_T(V, NV, DI, DO)                                                              \
   expert_scale_kernel<V, NV, DI, DO><<<grid, BLOCK, 0, st>>>(                                \
       (const V*)expert_x, expert_num_tokens, g.nle, g.max_recv, scale, g.row_vecs, g.chunks, \
