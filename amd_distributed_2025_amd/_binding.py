@@ -1,0 +1,147 @@
+"""The two ways the host layer reaches the C ABI of libmoe_a2a.so.
+
+`CtypesBinding` calls the exported functions directly (include/moe_a2a.h);
+`ExtBinding` goes through the torch extension of `csrc/moe_a2a_torch.cpp`, the
+binding idiom of the reference's submissions (all2all/hipv8.py:230-252). Both
+offer the same methods with the same arguments — tensors, sizes and the stream
+handle — and both end in the same kernels, so results are identical. Neither has
+a fallback: a missing library or a nonzero status raises.
+
+Capacities (`capacity_rows` of the C ABI) are taken from the tensors: the rows a
+row buffer and its meta buffer were allocated with.
+"""
+from __future__ import annotations
+
+import ctypes as C
+from typing import Optional
+
+import torch
+
+from . import _lib
+
+META_DIM = 5
+_DT = {torch.float16: _lib.F16, torch.bfloat16: _lib.BF16}
+
+
+def _ptr(t: Optional[torch.Tensor]):
+    return None if t is None else C.c_void_p(t.data_ptr())
+
+
+def _rows(buf: torch.Tensor, meta: torch.Tensor, hidden_dim: int) -> int:
+    return min(buf.numel() // max(hidden_dim, 1), meta.numel() // META_DIM)
+
+
+class CtypesBinding:
+    name = "ctypes"
+
+    def __init__(self):
+        _lib.load()
+
+    def version(self) -> str:
+        return _lib.load().moe_a2a_version().decode()
+
+    def dispatch_send(self, shape, x, indices, num_tokens, send_buf, send_meta, send_counts, send_slot, stream):
+        _lib.call("moe_a2a_dispatch_send", C.byref(shape), _ptr(x), _ptr(indices), num_tokens, _ptr(send_buf),
+                  _ptr(send_meta), _ptr(send_counts), _ptr(send_slot), C.c_void_p(stream))
+
+    def plan_send(self, shape, indices, num_tokens, rank_counts, rank_offsets, expert_counts, dst_slot,
+                  src_entry, stream):
+        _lib.call("moe_a2a_plan_send", C.byref(shape), _ptr(indices), num_tokens, _ptr(rank_counts),
+                  _ptr(rank_offsets), _ptr(expert_counts), _ptr(dst_slot), _ptr(src_entry), C.c_void_p(stream))
+
+    def dispatch_recv(self, shape, recv_buf, recv_meta, recv_counts, rows_hint, expert_num_tokens, expert_x,
+                      expert_meta, send_back_plan, stream):
+        capacity = _rows(recv_buf, recv_meta, shape.hidden_dim)
+        _lib.call("moe_a2a_dispatch_recv", C.byref(shape), _ptr(recv_buf), _ptr(recv_meta), _ptr(recv_counts),
+                  min(rows_hint, capacity), capacity, _ptr(expert_num_tokens), _ptr(expert_x), _ptr(expert_meta),
+                  _ptr(send_back_plan), C.c_void_p(stream))
+
+    def combine_send(self, shape, expert_y, expert_meta, expert_num_tokens, rows_hint, send_buf, send_meta,
+                     send_counts, send_back_plan, stream):
+        capacity = _rows(send_buf, send_meta, shape.hidden_dim)
+        _lib.call("moe_a2a_combine_send", C.byref(shape), _ptr(expert_y), _ptr(expert_meta),
+                  _ptr(expert_num_tokens), min(rows_hint, capacity), capacity, _ptr(send_buf), _ptr(send_meta),
+                  _ptr(send_counts), _ptr(send_back_plan), C.c_void_p(stream))
+
+    def combine_recv(self, shape, recv_buf, recv_meta, recv_counts, rows_hint, weights, num_tokens, out_tokens,
+                     accumulate, stream):
+        capacity = _rows(recv_buf, recv_meta, shape.hidden_dim)
+        _lib.call("moe_a2a_combine_recv", C.byref(shape), _ptr(recv_buf), _ptr(recv_meta), _ptr(recv_counts),
+                  min(rows_hint, capacity), capacity, _ptr(weights), num_tokens, _ptr(out_tokens),
+                  int(bool(accumulate)), _DT[out_tokens.dtype], C.c_void_p(stream))
+
+    def expert_scale(self, shape, expert_x, expert_num_tokens, rows_hint, expert_y, stream):
+        _lib.call("moe_a2a_expert_scale", C.byref(shape), _ptr(expert_x), _ptr(expert_num_tokens), rows_hint,
+                  _DT[expert_x.dtype], _DT[expert_y.dtype], _ptr(expert_y), C.c_void_p(stream))
+
+    def exchange_local(self, world_size, hidden_dim, send_buf, send_meta, send_counts, dst_rank, recv_buf,
+                       recv_meta, recv_counts, src_rank, rows_hint, stream):
+        _lib.call("moe_a2a_exchange_local", world_size, hidden_dim, _ptr(send_buf), _ptr(send_meta),
+                  _ptr(send_counts), dst_rank, _ptr(recv_buf), _ptr(recv_meta), _ptr(recv_counts), src_rank,
+                  rows_hint, _rows(send_buf, send_meta, hidden_dim), _rows(recv_buf, recv_meta, hidden_dim),
+                  C.c_void_p(stream))
+
+
+class ExtBinding:
+    name = "ext"
+
+    def __init__(self):
+        from . import _ext
+
+        self._m = _ext.load()
+
+    @staticmethod
+    def _shape(shape) -> list:
+        return [getattr(shape, f) for f, _ in _lib.Shape._fields_]
+
+    def version(self) -> str:
+        return self._m.a2a_version()
+
+    def dispatch_send(self, shape, x, indices, num_tokens, send_buf, send_meta, send_counts, send_slot, stream):
+        self._m.a2a_dispatch_send(self._shape(shape), x, indices, num_tokens, send_buf, send_meta, send_counts,
+                                  send_slot, stream)
+
+    def plan_send(self, shape, indices, num_tokens, rank_counts, rank_offsets, expert_counts, dst_slot,
+                  src_entry, stream):
+        self._m.a2a_plan_send(self._shape(shape), indices, num_tokens, rank_counts, rank_offsets, expert_counts,
+                              dst_slot, src_entry, stream)
+
+    def dispatch_recv(self, shape, recv_buf, recv_meta, recv_counts, rows_hint, expert_num_tokens, expert_x,
+                      expert_meta, send_back_plan, stream):
+        self._m.a2a_dispatch_recv(self._shape(shape), recv_buf, recv_meta, recv_counts, rows_hint,
+                                  expert_num_tokens, expert_x, expert_meta, send_back_plan, stream)
+
+    def combine_send(self, shape, expert_y, expert_meta, expert_num_tokens, rows_hint, send_buf, send_meta,
+                     send_counts, send_back_plan, stream):
+        self._m.a2a_combine_send(self._shape(shape), expert_y, expert_meta, expert_num_tokens, rows_hint,
+                                 send_buf, send_meta, send_counts, send_back_plan, stream)
+
+    def combine_recv(self, shape, recv_buf, recv_meta, recv_counts, rows_hint, weights, num_tokens, out_tokens,
+                     accumulate, stream):
+        self._m.a2a_combine_recv(self._shape(shape), recv_buf, recv_meta, recv_counts, rows_hint, weights,
+                                 num_tokens, out_tokens, bool(accumulate), stream)
+
+    def expert_scale(self, shape, expert_x, expert_num_tokens, rows_hint, expert_y, stream):
+        self._m.a2a_expert_scale(self._shape(shape), expert_x, expert_num_tokens, rows_hint, expert_y, stream)
+
+    def exchange_local(self, world_size, hidden_dim, send_buf, send_meta, send_counts, dst_rank, recv_buf,
+                       recv_meta, recv_counts, src_rank, rows_hint, stream):
+        self._m.a2a_exchange_local(world_size, hidden_dim, send_buf, send_meta, send_counts, dst_rank, recv_buf,
+                                   recv_meta, recv_counts, src_rank, rows_hint, stream)
+
+
+_BINDINGS = {}
+
+
+def get(name: str):
+    """`"ctypes"` or `"ext"`; bindings are created once."""
+    b = _BINDINGS.get(name)
+    if b is None:
+        if name == "ctypes":
+            b = CtypesBinding()
+        elif name == "ext":
+            b = ExtBinding()
+        else:
+            raise ValueError(f"unknown binding {name!r} (ctypes or ext)")
+        _BINDINGS[name] = b
+    return b

@@ -7,35 +7,35 @@
 accumulates into `out_tokens`. Each of the two is split into its send half and
 its receive half (`dispatch_send`/`dispatch_recv`, `combine_send`/
 `combine_recv`), because the exchange between the halves is not part of this
-library: an `exchange` object supplies it. `LocalWorld` is the one-GPU
-stand-in — it steps all ranks of a job in lockstep on one device and moves the
-segments with device copies.
+library: an `exchange` object supplies it through one method,
+`deliver(rank_object, phase, counts, buf, meta) -> (recv_counts, recv_buf,
+recv_meta, rows_hint)`. `LocalExchange` is the one-GPU stand-in for the
+reference's `all_to_all_single` calls: the ranks of a job run as threads of one
+process, meet in `deliver` as processes meet in a collective, and the segments
+move by device copies. `run_lockstep` starts such a job. `LocalWorld` steps all
+ranks of a job from one thread, half by half, with the same copies.
 
-All device work goes through the C ABI in `libmoe_a2a.so`; torch only owns
+All device work goes through the C ABI in `libmoe_a2a.so`, bound either with
+ctypes or through the torch extension (`binding="ext"`); torch only owns
 memory and streams. Buffers live in a per-object workspace allocated once, so
 the tensors returned by `dispatch` are views that stay valid until the next
 `dispatch` on the same object.
 """
 from __future__ import annotations
 
-import ctypes as C
-from typing import List, Optional, Sequence, Tuple
+import threading
+from typing import Callable, List, Optional, Sequence, Tuple
 
 import torch
 
-from . import _lib
-from .task import MoEConfig, RankTestData, dtype_name
+from . import _binding, _lib
+from .task import MoEConfig, RankTestData
 
 META_DIM = 5
-_DT = {"fp16": _lib.F16, "bf16": _lib.BF16}
 
 
-def _ptr(t: Optional[torch.Tensor]):
-    return None if t is None else C.c_void_p(t.data_ptr())
-
-
-def _stream(device) -> C.c_void_p:
-    return C.c_void_p(torch.cuda.current_stream(device).cuda_stream)
+def _stream(device) -> int:
+    return torch.cuda.current_stream(device).cuda_stream
 
 
 def _need(t: torch.Tensor, dtype: torch.dtype, device, what: str) -> torch.Tensor:
@@ -52,7 +52,7 @@ class HIPAllToAll:
     META_DIM = META_DIM  # global_exp, src_rank, src_token, src_k, pad
 
     def __init__(self, cfg: MoEConfig, rank: int, world_size: int, exchange=None, device=None,
-                 reuse_placement: bool = True):
+                 reuse_placement: bool = True, binding: str = "ctypes"):
         if cfg.num_experts % world_size:
             raise ValueError("num_experts must be a multiple of world_size")
         self.cfg = cfg
@@ -60,14 +60,14 @@ class HIPAllToAll:
         self.world_size = world_size
         self.num_local_experts = cfg.num_experts // world_size
         self.max_recv = cfg.max_num_tokens * world_size
-        self.exchange = exchange
+        # a job of one rank exchanges with itself; larger jobs need the object their ranks share
+        self.exchange = LocalExchange(1) if exchange is None and world_size == 1 else exchange
         self.device = torch.device("cuda", torch.cuda.current_device()) if device is None else torch.device(device)
         if self.device.type != "cuda":
             raise _lib.MoeA2AError("HIPAllToAll needs a GPU device; this path has no CPU fallback")
-        _lib.load()
+        self.binding = _binding.get(binding)  # raises if the native code has not been built
         self.shape = _lib.Shape(world_size, rank, cfg.num_experts, cfg.experts_per_token,
                                 cfg.hidden_dim, cfg.max_num_tokens)
-        self._shape_ref = C.byref(self.shape)
         # rows this rank can receive: every peer may route min(K, nle) entries of each token here
         self.max_rows_in = self.max_recv * min(cfg.experts_per_token, self.num_local_experts)
         self.max_rows_out = cfg.max_num_tokens * cfg.experts_per_token
@@ -116,8 +116,7 @@ class HIPAllToAll:
         buf = self._buf("send_buf", (self.max_rows_out, cfg.hidden_dim), cfg.in_dtype)
         meta = self._buf("send_meta", (self.max_rows_out, META_DIM), torch.int32)
         slots = self._buf("send_slot", (self.max_rows_out,), torch.int32) if want_slots else None
-        _lib.call("moe_a2a_dispatch_send", self._shape_ref, _ptr(dp_x), _ptr(indices), T,
-                  _ptr(buf), _ptr(meta), _ptr(counts), _ptr(slots), _stream(self.device))
+        self.binding.dispatch_send(self.shape, dp_x, indices, T, buf, meta, counts, slots, _stream(self.device))
         out = (counts, buf[:S], meta[:S])
         return out + (slots[:S],) if want_slots else out
 
@@ -135,8 +134,7 @@ class HIPAllToAll:
         ec = self._buf("plan_expert_counts", (cfg.num_experts,), torch.int32)
         ds = self._buf("plan_dst_slot", (self.max_rows_out,), torch.int32)
         se = self._buf("plan_src_entry", (self.max_rows_out,), torch.int32)
-        _lib.call("moe_a2a_plan_send", self._shape_ref, _ptr(indices), T, _ptr(rc), _ptr(ro), _ptr(ec),
-                  _ptr(ds), _ptr(se), _stream(self.device))
+        self.binding.plan_send(self.shape, indices, T, rc, ro, ec, ds, se, _stream(self.device))
         return rc, ro, ec, ds[:S], se[:S]
 
     def dispatch_recv(self, recv_counts, recv_buf, recv_meta, rows_hint: Optional[int] = None):
@@ -153,9 +151,8 @@ class HIPAllToAll:
         ex = self._buf("expert_x", (nle, self.max_recv, cfg.hidden_dim), cfg.in_dtype)
         em = self._buf("expert_meta", (nle, self.max_recv, META_DIM), torch.int32)
         plan = self._buf("send_back_plan", (2 * cfg.num_experts,), torch.int32) if self.reuse_placement else None
-        _lib.call("moe_a2a_dispatch_recv", self._shape_ref, _ptr(recv_buf), _ptr(recv_meta),
-                  _ptr(recv_counts), hint, capacity, _ptr(num), _ptr(ex), _ptr(em), _ptr(plan),
-                  _stream(self.device))
+        self.binding.dispatch_recv(self.shape, recv_buf, recv_meta, recv_counts, hint, num, ex, em, plan,
+                                   _stream(self.device))
         self._planned_for = None if plan is None else (em.data_ptr(), num.data_ptr())
         self._rows_in_hint = hint
         return num, ex, em
@@ -167,9 +164,7 @@ class HIPAllToAll:
         _need(expert_num_tokens, torch.int32, self.device, "expert_num_tokens")
         hint = self._default_rows_in(rows_hint)
         ey = self._buf("expert_y", tuple(expert_x.shape), cfg.out_dtype)
-        _lib.call("moe_a2a_expert_scale", self._shape_ref, _ptr(expert_x), _ptr(expert_num_tokens),
-                  hint, _DT[dtype_name(cfg.in_dtype)], _DT[dtype_name(cfg.out_dtype)], _ptr(ey),
-                  _stream(self.device))
+        self.binding.expert_scale(self.shape, expert_x, expert_num_tokens, hint, ey, _stream(self.device))
         return ey
 
     def combine_send(self, expert_meta, expert_y, expert_num_tokens, rows_hint: Optional[int] = None):
@@ -192,9 +187,8 @@ class HIPAllToAll:
         plan = None
         if self._planned_for == (expert_meta.data_ptr(), expert_num_tokens.data_ptr()):
             plan = self._ws["send_back_plan"]
-        _lib.call("moe_a2a_combine_send", self._shape_ref, _ptr(expert_y), _ptr(expert_meta),
-                  _ptr(expert_num_tokens), min(hint, self.max_rows_in), self.max_rows_in, _ptr(buf),
-                  _ptr(meta), _ptr(counts), _ptr(plan), _stream(self.device))
+        self.binding.combine_send(self.shape, expert_y, expert_meta, expert_num_tokens,
+                                  min(hint, self.max_rows_in), buf, meta, counts, plan, _stream(self.device))
         return counts, buf, meta
 
     def combine_recv(self, out_tokens, weights, ret_counts, ret_buf, ret_meta, accumulate: bool = True):
@@ -212,9 +206,8 @@ class HIPAllToAll:
             raise ValueError("combine: out_tokens must hold num_tokens rows of hidden_dim")
         capacity = min(ret_buf.shape[0], ret_meta.shape[0])
         hint = min(capacity, T * cfg.experts_per_token)
-        _lib.call("moe_a2a_combine_recv", self._shape_ref, _ptr(ret_buf), _ptr(ret_meta),
-                  _ptr(ret_counts), hint, capacity, _ptr(weights), T, _ptr(out_tokens), int(bool(accumulate)),
-                  _DT[dtype_name(cfg.out_dtype)], _stream(self.device))
+        self.binding.combine_recv(self.shape, ret_buf, ret_meta, ret_counts, hint, weights, T, out_tokens,
+                                  accumulate, _stream(self.device))
         return out_tokens
 
     def _default_rows_in(self, rows_hint):
@@ -227,7 +220,8 @@ class HIPAllToAll:
     def dispatch(self, dp_x: torch.Tensor, indices: torch.Tensor):
         """all2all/reference.py:68-148 with the exchange delegated to `self.exchange`."""
         if self.exchange is None:
-            raise RuntimeError("dispatch() needs an exchange; use the halves or LocalWorld")
+            raise RuntimeError("dispatch() of a job with several ranks needs the exchange its ranks share "
+                               "(LocalExchange on one GPU); or use the halves, or LocalWorld")
         counts, buf, meta = self.dispatch_send(dp_x, indices)
         rc, rb, rm, hint = self.exchange.deliver(self, "dispatch", counts, buf, meta)
         return self.dispatch_recv(rc, rb, rm, hint)
@@ -235,7 +229,8 @@ class HIPAllToAll:
     def combine(self, out_tokens, weights, expert_meta, expert_y, expert_num_tokens):
         """all2all/reference.py:151-234 with the exchange delegated to `self.exchange`."""
         if self.exchange is None:
-            raise RuntimeError("combine() needs an exchange; use the halves or LocalWorld")
+            raise RuntimeError("combine() of a job with several ranks needs the exchange its ranks share "
+                               "(LocalExchange on one GPU); or use the halves, or LocalWorld")
         counts, buf, meta = self.combine_send(expert_meta, expert_y, expert_num_tokens)
         rc, rb, rm, _ = self.exchange.deliver(self, "combine", counts, buf, meta)
         return self.combine_recv(out_tokens, weights, rc, rb, rm, accumulate=True)
@@ -245,12 +240,83 @@ def exchange_leg(src: HIPAllToAll, dst: HIPAllToAll, send_counts, send_buf, send
                  recv_counts, recv_buf, recv_meta, rows_hint: int) -> None:
     """One source->destination leg of an exchange as a device copy. The copy stays inside the
     rows the four buffers were allocated with, whatever the counts say."""
-    send_capacity = min(send_buf.shape[0], send_meta.shape[0])
-    recv_capacity = min(recv_buf.shape[0], recv_meta.shape[0])
-    _lib.call("moe_a2a_exchange_local", src.world_size, src.cfg.hidden_dim, _ptr(send_buf),
-              _ptr(send_meta), _ptr(send_counts), dst.rank, _ptr(recv_buf), _ptr(recv_meta),
-              _ptr(recv_counts), src.rank, int(rows_hint), send_capacity, recv_capacity,
-              _stream(src.device))
+    src.binding.exchange_local(src.world_size, src.cfg.hidden_dim, send_buf, send_meta, send_counts, dst.rank,
+                               recv_buf, recv_meta, recv_counts, src.rank, int(rows_hint), _stream(src.device))
+
+
+class LocalExchange:
+    """The exchange of a job whose ranks share one GPU and one process: stand-in for the
+    `all_to_all_single` calls of all2all/reference.py:91,107-119 (dispatch) and :185,210-222
+    (combine).
+
+    Every rank runs in a thread of its own and calls `dispatch()` / `combine()` as a process
+    of the reference would; `deliver` is where they meet. Each rank posts what it sends and
+    waits for the others (as in a collective), then copies the segments addressed to it out of
+    its peers' send buffers with `moe_a2a_exchange_local`, and waits again so that no peer
+    reuses a send buffer before every copy out of it has been launched. All launches go to the
+    callers' current stream, which the ranks must share (the default stream does), so launch
+    order is execution order.
+
+    `exact_hints=True` reads the counts back (one host synchronisation per call, as the
+    reference's `.tolist()` at reference.py:110-111) and sizes every launch exactly; otherwise
+    launches are sized for the largest segment the buffers can hold and nothing waits for the
+    device.
+    """
+
+    def __init__(self, world_size: int, exact_hints: bool = False, timeout: float = 120.0):
+        self.world_size = world_size
+        self.exact_hints = exact_hints
+        self._posted: List[Optional[tuple]] = [None] * world_size
+        # a rank that fails leaves the others waiting: the time-out turns that into an error
+        self._barrier = threading.Barrier(world_size, timeout=timeout)
+
+    def deliver(self, a: "HIPAllToAll", phase: str, counts, buf, meta):
+        W = self.world_size
+        if a.world_size != W:
+            raise ValueError("this exchange serves a job of another size")
+        self._posted[a.rank] = (a, counts, buf, meta)
+        self._barrier.wait()  # every rank has launched its send half
+        posted = list(self._posted)
+        rc, rb, rm = a.inbound_buffers(phase)
+        sent_here = torch.stack([p[1] for p in posted])[:, a.rank]  # rows each source holds for this rank
+        rc.copy_(sent_here)
+        host = sent_here.cpu().tolist() if self.exact_hints else None
+        bound = min(rb.shape[0], rm.shape[0])
+        for s, (src, sc, sb, sm) in enumerate(posted):
+            hint = host[s] if host is not None else min(bound, sb.shape[0])
+            if hint > 0:
+                exchange_leg(src, a, sc, sb, sm, rc, rb, rm, hint)
+        self._barrier.wait()  # every copy out of every send buffer has been launched
+        return rc, rb, rm, (sum(host) if host is not None else None)
+
+
+def run_lockstep(world_size: int, rank_main: Callable[[int, LocalExchange], object],
+                 exact_hints: bool = False, device=None) -> list:
+    """Run `rank_main(rank, exchange)` for every rank of a job, one thread per rank on one
+    GPU, and return the results in rank order: what a launcher with one process per GPU does
+    for the reference. The first exception of any rank is raised again here."""
+    exchange = LocalExchange(world_size, exact_hints=exact_hints)
+    results: list = [None] * world_size
+    errors: list = [None] * world_size
+    dev = torch.device("cuda", torch.cuda.current_device()) if device is None else torch.device(device)
+
+    def body(r: int):
+        try:
+            with torch.cuda.device(dev):
+                results[r] = rank_main(r, exchange)
+        except BaseException as e:  # noqa: BLE001 - handed to the caller below
+            errors[r] = e
+            exchange._barrier.abort()  # release the ranks waiting for this one
+
+    threads = [threading.Thread(target=body, args=(r,), name=f"rank{r}") for r in range(world_size)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    real = [e for e in errors if e is not None and not isinstance(e, threading.BrokenBarrierError)]
+    if real or any(errors):
+        raise (real or [e for e in errors if e is not None])[0]
+    return results
 
 
 class LocalWorld:
@@ -258,10 +324,10 @@ class LocalWorld:
     device copies (stand-in for all2all/reference.py:91,107-119,185,210-222)."""
 
     def __init__(self, cfg: MoEConfig, world_size: int, device=None, exact_hints: bool = True,
-                 reuse_placement: bool = True):
+                 reuse_placement: bool = True, binding: str = "ctypes"):
         self.cfg, self.world_size = cfg, world_size
-        self.ranks = [HIPAllToAll(cfg, r, world_size, device=device, reuse_placement=reuse_placement)
-                      for r in range(world_size)]
+        self.ranks = [HIPAllToAll(cfg, r, world_size, device=device, reuse_placement=reuse_placement,
+                                  binding=binding) for r in range(world_size)]
         self.device = self.ranks[0].device
         # True: read the counts back to size every launch exactly (synchronises the host);
         # False: size for the worst case; "last": reuse what the previous run read back, for

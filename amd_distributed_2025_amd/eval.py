@@ -101,20 +101,30 @@ def geometric_mean(values: Sequence[float]) -> float:
 
 def run_tests(spec: Dict, device, reference: Optional[Callable[[input_t], output_t]] = None,
               log=print) -> bool:
-    from .submission import custom_kernel, set_peer_inputs
+    """Every job of the test list: the job is stepped once (all ranks together, as the
+    reference's harness has all ranks call `custom_kernel` at the same time) and every rank's
+    output is checked; rank 0 is also asked for through `custom_kernel` itself."""
+    from .submission import custom_kernel, custom_kernel_job, set_peer_inputs
 
     all_ok = True
     for n, job in enumerate(spec["tests"]):
         world = job_inputs(job, device)
-        set_peer_inputs(world)
-        for data in world:
-            out = custom_kernel(data)
+        outs = custom_kernel_job(world)
+        job_ok = True
+        for data, out in zip(world, outs):
             ok, msg = check_implementation(None if reference is None else reference(data), out, data)
             if not ok:
-                all_ok = False
+                job_ok = False
                 log(f"test {n} {job} rank {data[2]}: FAIL {msg}")
-        log(f"test {n} {job}: {'checked' if all_ok else 'see failures above'}")
-    set_peer_inputs(None)
+        set_peer_inputs(world)
+        try:
+            if not torch.equal(custom_kernel(world[0]), outs[0]):
+                job_ok = False
+                log(f"test {n} {job} rank 0: FAIL custom_kernel(data) differs from the job's step")
+        finally:
+            set_peer_inputs(None)
+        log(f"test {n} {job}: {'checked' if job_ok else 'see failures above'}")
+        all_ok = all_ok and job_ok
     return all_ok
 
 

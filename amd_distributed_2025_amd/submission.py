@@ -39,6 +39,20 @@ def _world_for(cfg: MoEConfig, world_size: int, device: torch.device) -> LocalWo
     return w
 
 
+def custom_kernel_job(inputs: Sequence[input_t]) -> list:
+    """Every rank's `custom_kernel` result from ONE step of the job: what W processes calling
+    `custom_kernel` at the same time produce together. `inputs[r]` is rank r's tuple."""
+    cfg, first, _, world_size = inputs[0]
+    device = first.x.device
+    if device.type != "cuda":
+        raise RuntimeError("custom_kernel needs its inputs on a GPU; this path has no CPU fallback")
+    if len(inputs) != world_size:
+        raise ValueError(f"a job of world_size={world_size} needs {world_size} inputs, got {len(inputs)}")
+    with torch.cuda.device(device):
+        ys = _world_for(cfg, world_size, device).run([d[1].to(device) for d in inputs])
+        return [y.clone() for y in ys]
+
+
 def custom_kernel(data: input_t) -> output_t:
     cfg, rank_data, rank, world_size = data
     device = rank_data.x.device

@@ -161,3 +161,36 @@ def test_workload_generators():
     hot5 = np.bincount(skew[5][1].indices.numpy().ravel(), minlength=256).argmax()
     assert hot0 == hot5 == np.bincount(ids, minlength=256).argmax()
     assert len(TASK_YML_TESTS) == 9 and len(TASK_YML_BENCHMARKS) == 5
+
+
+def test_torch_extension_wraps_every_entry_point():
+    """The module built by load_inline loads without a GPU, reports the library's version, has
+    one wrapper per entry point that launches work, and refuses tensors that are not on a GPU
+    before anything reaches the library."""
+    from amd_distributed_2025_amd import _ext
+    from amd_distributed_2025_amd.build import EXT_FUNCTIONS
+
+    m = _ext.load()
+    assert m.a2a_version() == _lib.load().moe_a2a_version().decode()
+    wrapped = {"moe_" + f for f in EXT_FUNCTIONS}
+    assert wrapped == set(declared_functions()) - {"moe_a2a_strerror"}
+    source = (ROOT / "amd_distributed_2025_amd" / "csrc" / "moe_a2a_torch.cpp").read_text()
+    for f in EXT_FUNCTIONS:
+        assert hasattr(m, f), f
+        assert "moe_" + f + "(" in source, f  # every wrapper ends in the C ABI call of its name
+    x = torch.zeros(4, 16, dtype=torch.bfloat16)
+    idx = torch.zeros(4, 2, dtype=torch.int32)
+    with pytest.raises(RuntimeError, match="x: must be a GPU tensor"):
+        m.a2a_dispatch_send([1, 0, 8, 2, 16, 4], x, idx, 4, torch.zeros(8, 16, dtype=torch.bfloat16),
+                            torch.zeros(8, 5, dtype=torch.int32), torch.zeros(1, dtype=torch.int32), None, 0)
+    with pytest.raises(RuntimeError, match="shape: expected"):
+        m.a2a_dispatch_send([1, 0, 8], x, idx, 4, x, idx, idx, None, 0)
+
+
+def test_unknown_binding_is_refused():
+    from amd_distributed_2025_amd import _binding
+
+    with pytest.raises(ValueError, match="unknown binding"):
+        _binding.get("cffi")
+    assert _binding.get("ctypes").version().startswith("moe_a2a")
+    assert _binding.get("ext").version() == _binding.get("ctypes").version()

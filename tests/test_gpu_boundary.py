@@ -1,0 +1,236 @@
+"""The drop-in boundary on a real GPU: the reference's class surface
+(`dispatch` / `combine`, all2all/reference.py:68,151) driven exactly as
+`ref_kernel` drives it (reference.py:259-272), the torch-extension binding
+against the ctypes binding, and the oracle's 16-bit arithmetic against torch's
+own on the device the reference runs on."""
+import numpy as np
+import pytest
+import torch
+
+from amd_distributed_2025_amd import HIPAllToAll, LocalWorld, WORKLOADS, generate_world
+from amd_distributed_2025_amd.all2all import LocalExchange, run_lockstep
+from amd_distributed_2025_amd.task import DTYPES, MoEConfig
+from oracle import moe_a2a_oracle as orc
+from tests.helpers import bits, from_bits, run_oracle
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def ref_kernel_body(ata, cfg, rank_data, rank, seen):
+    """The statements of all2all/reference.py:259-272 with the class under test."""
+    expert_num, expert_x, expert_meta = ata.dispatch(rank_data.x, rank_data.indices)
+    seen.update(expert_num=expert_num, expert_x=expert_x, expert_meta=expert_meta)
+    expert_y = expert_x.to(cfg.out_dtype) * (1 + rank)
+    y = torch.zeros(cfg.max_num_tokens, cfg.hidden_dim, dtype=cfg.out_dtype, device=rank_data.x.device)
+    ata.combine(y, rank_data.weights, expert_meta, expert_y, expert_num)
+    return y[: rank_data.num_tokens]
+
+
+@pytest.mark.parametrize("name,binding", [("C1", "ctypes"), ("C2", "ctypes"), ("C2", "ext"), ("C3", "ctypes")])
+@pytest.mark.parametrize("exact_hints", [False, True])
+def test_reference_class_surface_runs_ref_kernel(name, binding, exact_hints):
+    """Only `dispatch(dp_x, indices)` and `combine(out_tokens, weights, expert_meta, expert_y,
+    expert_num_tokens)` are called, one thread per rank as the reference has one process per
+    rank; every rank's result and the three returned layouts are checked."""
+    print(f"class surface {name} {binding} exact_hints={exact_hints}", flush=True)
+    world = generate_world(WORKLOADS[name], 2025)
+    cfg, W = world[0][0], len(world)
+    nle, max_recv = cfg.num_experts // W, cfg.max_num_tokens * W
+    dev = [d.to(DEV) for _, d, _, _ in world]
+    seen = [dict() for _ in range(W)]
+
+    def rank_main(rank, exchange):
+        ata = HIPAllToAll(cfg, rank, W, exchange=exchange, device=DEV, binding=binding)
+        y = ref_kernel_body(ata, cfg, dev[rank], rank, seen[rank])
+        torch.cuda.synchronize()
+        return y.clone(), {k: v.clone() for k, v in seen[rank].items()}
+
+    results = run_lockstep(W, rank_main, exact_hints=exact_hints, device=DEV)
+    want = run_oracle(world)
+    for r, (y, layouts) in enumerate(results):
+        num, ex, em = layouts["expert_num"], layouts["expert_x"], layouts["expert_meta"]
+        # the layouts of all2all/reference.py:123-136,148
+        assert num.shape == (nle,) and num.dtype == torch.int32
+        assert ex.shape == (nle, max_recv, cfg.hidden_dim) and ex.dtype == cfg.in_dtype
+        assert em.shape == (nle, max_recv, 5) and em.dtype == torch.int32
+        assert y.shape == (dev[r].num_tokens, cfg.hidden_dim) and y.dtype == cfg.out_dtype
+        cnt = num.cpu().numpy()
+        assert np.array_equal(cnt, want[r].expert_num_tokens), r
+        rows = torch.cat([ex[le, : int(cnt[le])] for le in range(nle)])
+        metas = torch.cat([em[le, : int(cnt[le])] for le in range(nle)])
+        assert np.array_equal(bits(rows), want[r].expert_rows), r
+        assert np.array_equal(metas.cpu().numpy(), want[r].expert_meta_rows), r
+        assert np.array_equal(bits(y), want[r].y), f"rank {r}: combined rows differ from the oracle"
+
+
+def test_single_rank_job_needs_no_exchange_object():
+    world = generate_world(WORKLOADS["C1"], 11)
+    cfg, d = world[0][0], world[0][1].to(DEV)
+    y = ref_kernel_body(HIPAllToAll(cfg, 0, 1, device=DEV), cfg, d, 0, {})
+    torch.cuda.synchronize()
+    assert np.array_equal(bits(y), run_oracle(world)[0].y)
+
+
+def test_several_ranks_without_exchange_say_what_is_missing():
+    world = generate_world(WORKLOADS["C2"], 11)
+    cfg, d = world[0][0], world[0][1].to(DEV)
+    with pytest.raises(RuntimeError, match="exchange"):
+        HIPAllToAll(cfg, 0, 8, device=DEV).dispatch(d.x, d.indices)
+
+
+def test_a_failing_rank_does_not_leave_the_others_waiting():
+    world = generate_world(WORKLOADS["C2"], 3)
+    cfg, W = world[0][0], len(world)
+    dev = [d.to(DEV) for _, d, _, _ in world]
+
+    def rank_main(rank, exchange):
+        if rank == 3:
+            raise ValueError("rank 3 gives up")
+        return HIPAllToAll(cfg, rank, W, exchange=exchange, device=DEV).dispatch(dev[rank].x, dev[rank].indices)
+
+    with pytest.raises(ValueError, match="rank 3 gives up"):
+        run_lockstep(W, rank_main, device=DEV)
+    torch.cuda.synchronize()
+
+
+TRACE_KEYS = ("send_counts", "send_buf", "send_meta", "send_slot", "recv_counts", "expert_num_tokens",
+              "back_counts", "ret_counts", "y")
+
+
+@pytest.mark.parametrize("name", ["C2", "C3"])
+def test_extension_binding_gives_the_bits_of_the_ctypes_binding(name):
+    """The whole job through the torch extension (torch::Tensor wrappers built by load_inline)
+    and through ctypes: every intermediate of every rank is identical, and equals the oracle."""
+    print(f"extension vs ctypes {name}", flush=True)
+    world = generate_world(WORKLOADS[name], 77)
+    cfg, W = world[0][0], len(world)
+    dev = [d.to(DEV) for _, d, _, _ in world]
+    via_ext = LocalWorld(cfg, W, device=DEV, binding="ext")
+    via_ctypes = LocalWorld(cfg, W, device=DEV, binding="ctypes")
+    assert via_ext.ranks[0].binding.name == "ext" and via_ctypes.ranks[0].binding.name == "ctypes"
+    ys_e = via_ext.run(dev)
+    ys_c = via_ctypes.run(dev)
+    torch.cuda.synchronize()
+    want = run_oracle(world)
+    for r in range(W):
+        e, c = via_ext.trace[r], via_ctypes.trace[r]
+        S = dev[r].num_tokens * cfg.experts_per_token
+        R = int(c["recv_counts"].sum().item())
+        for key in TRACE_KEYS:
+            assert torch.equal(e[key], c[key]), (r, key)
+        for key, n in (("recv_buf", R), ("recv_meta", R), ("back_buf", R), ("back_meta", R),
+                       ("ret_buf", S), ("ret_meta", S)):
+            assert torch.equal(e[key][:n], c[key][:n]), (r, key)
+        cnt = c["expert_num_tokens"].cpu().numpy()
+        for le in range(cnt.size):
+            n = int(cnt[le])
+            for key in ("expert_x", "expert_meta", "expert_y"):
+                assert torch.equal(e[key][le, :n], c[key][le, :n]), (r, key, le)
+        assert torch.equal(ys_e[r], ys_c[r])
+        assert np.array_equal(bits(ys_e[r]), want[r].y)
+    # the explicit send plan through the extension
+    rc, ro, ec, dst, src = via_ext.ranks[0].plan_send(dev[0].indices)
+    rc2, ro2, ec2, dst2, src2 = via_ctypes.ranks[0].plan_send(dev[0].indices)
+    torch.cuda.synchronize()
+    for a, b in ((rc, rc2), (ro, ro2), (ec, ec2), (dst, dst2), (src, src2)):
+        assert torch.equal(a, b)
+
+
+def test_extension_checks_its_tensors_before_launching():
+    from amd_distributed_2025_amd import _ext
+
+    m = _ext.load()
+    shape = [1, 0, 4, 2, 64, 8]
+    T, K, H = 8, 2, 64
+    x = torch.zeros(T, H, dtype=torch.bfloat16, device=DEV)
+    idx = torch.zeros(T, K, dtype=torch.int32, device=DEV)
+    buf = torch.zeros(T * K, H, dtype=torch.bfloat16, device=DEV)
+    meta = torch.zeros(T * K, 5, dtype=torch.int32, device=DEV)
+    counts = torch.zeros(1, dtype=torch.int32, device=DEV)
+    st = torch.cuda.current_stream().cuda_stream
+    m.a2a_dispatch_send(shape, x, idx, T, buf, meta, counts, None, st)  # the good call
+    with pytest.raises(RuntimeError, match="indices: expected Int"):
+        m.a2a_dispatch_send(shape, x, idx.long(), T, buf, meta, counts, None, st)
+    with pytest.raises(RuntimeError, match="x: must be contiguous"):
+        m.a2a_dispatch_send(shape, torch.zeros(H, T, dtype=torch.bfloat16, device=DEV).t(), idx, T, buf, meta,
+                            counts, None, st)
+    with pytest.raises(RuntimeError, match="send_buf: holds"):
+        m.a2a_dispatch_send(shape, x, idx, T, buf[: T * K - 1], meta, counts, None, st)
+    with pytest.raises(RuntimeError, match="send_buf: expected BFloat16"):
+        m.a2a_dispatch_send(shape, x, idx, T, buf.to(torch.float16), meta, counts, None, st)
+    with pytest.raises(RuntimeError, match="x: token rows must be float16 or bfloat16"):
+        m.a2a_dispatch_send(shape, x.float(), idx, T, buf, meta, counts, None, st)
+    with pytest.raises(RuntimeError, match="send_meta: must be a GPU tensor"):
+        m.a2a_dispatch_send(shape, x, idx, T, buf, meta.cpu(), counts, None, st)
+    with pytest.raises(RuntimeError, match="status -1"):  # the library's own argument check
+        m.a2a_dispatch_send([1, 0, 4, 2, 64, 4], x, idx, T, buf, meta, counts, None, st)
+    torch.cuda.synchronize()
+
+
+# ----------------------------------------------------------------------------- arithmetic on the device
+
+
+def halfway_cases(name: str, n: int, rng) -> tuple:
+    """Pairs (a, b) of 16-bit values with a + b exactly halfway between two neighbours of a:
+    only round-to-nearest-EVEN after the addition gives the reference's bits."""
+    if name == "bf16":
+        mant_bits, exps = 7, rng.integers(-20, 60, n)
+    else:
+        mant_bits, exps = 10, rng.integers(-8, 10, n)
+    mant = rng.integers(0, 1 << mant_bits, n)
+    a = (1.0 + mant / float(1 << mant_bits)) * np.exp2(exps.astype(np.float64))
+    b = np.exp2(exps.astype(np.float64) - mant_bits - 1)  # half a unit in the last place of a
+    a16 = orc.f32_to_b16(a.astype(np.float32), name)
+    b16 = orc.f32_to_b16(b.astype(np.float32), name)
+    assert np.array_equal(orc.b16_to_f32(a16, name), a.astype(np.float32))  # both exact in 16 bits
+    assert np.array_equal(orc.b16_to_f32(b16, name), b.astype(np.float32))
+    return a16, b16
+
+
+@pytest.mark.parametrize("name", ["bf16", "fp16"])
+def test_oracle_accumulate_equals_torch_on_the_device(name):
+    """all2all/reference.py:232 as torch executes it on the GPU — `y16[t] += row.float() * w`
+    in a 16-bit tensor — for every 16-bit pattern as first addend, random second addends,
+    weights that force roundings, and exact ties, against the oracle's `combine_recv`."""
+    dt = DTYPES[name]
+    rng = np.random.default_rng(5)
+    H = 65536
+    allbits = np.arange(H, dtype=np.uint32).astype(np.uint16)
+    second = orc.f32_to_b16((rng.standard_normal(H) * 3).astype(np.float32), name)
+    tie_a, tie_b = halfway_cases(name, H, rng)
+    # token 0: every pattern, then a random addend; token 1: ties with unit weights; token 2: one addend
+    rows = np.stack([allbits, second, tie_a, tie_b, second])
+    meta = np.array([[0, 0, 0, 0, 0], [0, 0, 0, 1, 0], [0, 0, 1, 0, 0], [0, 0, 1, 1, 0], [0, 0, 2, 1, 0]], np.int32)
+    w = np.array([[1.0 + 2.0 ** -7, 0.3], [1.0, 1.0], [0.0, 0.7]], np.float32)
+    want = orc.combine_recv(rows, meta, w, 3, name)
+
+    recv = from_bits(rows, dt).to(DEV)
+    weights = torch.from_numpy(w).to(DEV)
+    y = torch.zeros(3, H, dtype=dt, device=DEV)
+    for i in range(rows.shape[0]):  # the loop of reference.py:227-232
+        src_token, src_k = int(meta[i, 2]), int(meta[i, 3])
+        weight = weights[src_token, src_k]
+        y[src_token] += recv[i].to(torch.float32) * weight
+    torch.cuda.synchronize()
+    got = bits(y)
+    nan = np.isnan(orc.b16_to_f32(want, name))
+    assert np.array_equal(got[~nan], want[~nan])
+    assert np.isnan(orc.b16_to_f32(got[nan], name)).all()
+    # the ties really are ties: adding in float32 and rounding the other way changes bits
+    exact = orc.b16_to_f32(tie_a, name) + orc.b16_to_f32(tie_b, name)
+    assert np.array_equal(orc.b16_to_f32(want[1], name) != exact, np.ones(H, bool))
+
+
+@pytest.mark.parametrize("name_in,name_out", [("bf16", "bf16"), ("fp16", "fp16"), ("fp16", "bf16"), ("bf16", "fp16")])
+def test_oracle_expert_scale_equals_torch_on_the_device(name_in, name_out):
+    """all2all/reference.py:262, `expert_x.to(out_dtype) * (1 + rank)`, as torch executes it on
+    the GPU, for every 16-bit pattern and every rank of an 8-rank job."""
+    allbits = np.arange(65536, dtype=np.uint32).astype(np.uint16)
+    x = from_bits(allbits, DTYPES[name_in]).to(DEV)
+    for rank in range(8):
+        got = bits(x.to(DTYPES[name_out]) * (1 + rank))
+        want = orc.expert_scale(allbits, rank, name_in, name_out)
+        nan = np.isnan(orc.b16_to_f32(want, name_out))
+        assert np.array_equal(got[~nan], want[~nan]), rank
+        assert np.isnan(orc.b16_to_f32(got[nan], name_out)).all(), rank
