@@ -24,9 +24,17 @@
 #include <hip/hip_fp16.h>
 #include <stdint.h>
 #include <limits.h>
+#include <mutex>
 #include <type_traits>
 
 #include "moe_a2a.h"
+
+// Device memory of moe_a2a_dispatch_recv_static: the send-back plan of one call, held by the
+// library so that the caller brings no buffer for it. Every GPU the library runs on has its own
+// copy at its own address; host code reaches it only through the address that
+// hipGetSymbolAddress returned for that GPU (static_plan_buffer below), never through this name.
+#define MOE_A2A_STATIC_PLAN_EXPERTS 4096  /* world_size <= 64 times num_local_experts <= 64 */
+static __device__ __align__(256) int32_t scratch[2 * MOE_A2A_STATIC_PLAN_EXPERTS];
 
 namespace {
 
@@ -1647,6 +1655,24 @@ bool plan_supported(const moe_a2a_shape* s) {
   return s->world_size <= 64 && s->num_experts / s->world_size <= 64;
 }
 
+// Address of `scratch` on the GPU that is current for the calling thread, looked up once per
+// GPU with that GPU current and kept. Returns nullptr if the runtime cannot name it.
+constexpr int MAX_GPUS = 64;
+std::mutex static_plan_mutex;
+int32_t* static_plan_address[MAX_GPUS] = {};
+
+int32_t* static_plan_buffer() {
+  int gpu = -1;
+  if (hipGetDevice(&gpu) != hipSuccess || gpu < 0 || gpu >= MAX_GPUS) return nullptr;
+  std::lock_guard<std::mutex> lock(static_plan_mutex);
+  if (!static_plan_address[gpu]) {
+    void* p = nullptr;
+    if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess) return nullptr;
+    static_plan_address[gpu] = static_cast<int32_t*>(p);
+  }
+  return static_plan_address[gpu];
+}
+
 // W counts, each cut to `capacity_rows` on the device, must add up inside an int.
 bool counts_fit(long long capacity_rows, int world_size) {
   return capacity_rows * world_size <= INT_MAX;
@@ -1661,7 +1687,7 @@ long long group_items(long long rows, const Geometry& g) {
 
 extern "C" {
 
-const char* moe_a2a_version(void) { return "moe_a2a 0.3 gfx950"; }
+const char* moe_a2a_version(void) { return "moe_a2a 0.4 gfx950"; }
 
 const char* moe_a2a_strerror(int status) {
   switch (status) {
@@ -1669,6 +1695,9 @@ const char* moe_a2a_strerror(int status) {
     case MOE_A2A_EINVAL: return "invalid argument (null pointer, bad shape or unsupported size)";
     case MOE_A2A_EALIGN: return "row buffer is not aligned to its 2-byte elements";
     case MOE_A2A_ELAUNCH: return "kernel launch failed";
+    case MOE_A2A_ESCRATCH:
+      return "shape beyond the library's static buffer (world_size <= 64 and num_local_experts <= 64), "
+             "or the buffer's address is unavailable";
     default: return "unknown status";
   }
 }
@@ -1782,6 +1811,24 @@ int moe_a2a_dispatch_recv(const moe_a2a_shape* s, const void* recv_buf, const in
 #undef LAUNCH
 #undef LAUNCH_P
   return launch_status();
+}
+
+int moe_a2a_dispatch_recv_static(const moe_a2a_shape* s, const void* recv_buf,
+                                 const int32_t* recv_meta, const int32_t* recv_counts,
+                                 int32_t rows_hint, int32_t capacity_rows, int32_t* expert_num_tokens,
+                                 void* expert_x, int32_t* expert_meta,
+                                 const int32_t** send_back_plan, void* stream) {
+  if (!shape_ok(s) || !send_back_plan) return MOE_A2A_EINVAL;
+  *send_back_plan = nullptr;
+  // the plan needs a lane per source rank and per local expert, and 2 * num_experts ints
+  if (!plan_supported(s) || s->num_experts > MOE_A2A_STATIC_PLAN_EXPERTS) return MOE_A2A_ESCRATCH;
+  int32_t* plan = static_plan_buffer();
+  if (!plan) return MOE_A2A_ESCRATCH;
+  // every int of the plan that this shape uses is written by the call: nothing to clear
+  const int rc = moe_a2a_dispatch_recv(s, recv_buf, recv_meta, recv_counts, rows_hint, capacity_rows,
+                                       expert_num_tokens, expert_x, expert_meta, plan, stream);
+  if (rc == MOE_A2A_OK) *send_back_plan = plan;
+  return rc;
 }
 
 int moe_a2a_combine_send(const moe_a2a_shape* s, const void* expert_y, const int32_t* expert_meta,

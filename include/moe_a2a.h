@@ -52,6 +52,7 @@ extern "C" {
 #define MOE_A2A_EINVAL (-1)   /* bad size / null pointer / unsupported value */
 #define MOE_A2A_EALIGN (-2)   /* a row buffer is not 2-byte aligned */
 #define MOE_A2A_ELAUNCH (-3)  /* hipGetLastError() != hipSuccess after launch */
+#define MOE_A2A_ESCRATCH (-4) /* shape beyond the library's static buffer         */
 
 /* Static shape of one rank's problem (reference: MoEConfig,
  * all2all/reference.py:10-17, and PyTorchAllToAll.__init__, :58-65). */
@@ -65,7 +66,7 @@ typedef struct moe_a2a_shape {
 } moe_a2a_shape;
 
 /* Library version / build probe. Returns a static string such as
- * "moe_a2a 0.3 gfx950"; the number changes with the ABI. Never NULL. */
+ * "moe_a2a 0.4 gfx950"; the number changes with the ABI. Never NULL. */
 const char* moe_a2a_version(void);
 
 /* Human-readable text for a status code. Never NULL. */
@@ -149,6 +150,38 @@ int moe_a2a_dispatch_recv(const moe_a2a_shape* shape, const void* recv_buf,
                           int32_t* expert_num_tokens, void* expert_x,
                           int32_t* expert_meta, int32_t* send_back_plan,
                           void* stream);
+
+/*
+ * moe_a2a_dispatch_recv with the send-back plan kept in device memory that the
+ * library owns, for callers that cannot allocate: code under HIP graph
+ * capture, serving loops and harnesses that must not call hipMalloc. It has no
+ * counterpart in the reference. Same arguments, results and kernels as
+ * moe_a2a_dispatch_recv, except that the plan is not brought by the caller:
+ *
+ *   send_back_plan  host pointer, out: where the call left the plan (a device
+ *                   address inside the library's static buffer), to be handed
+ *                   to moe_a2a_combine_send as its send_back_plan under the
+ *                   same rule as a caller-owned plan. NULL on any error.
+ *
+ * The call allocates and frees nothing and clears nothing (every int of the
+ * plan that the shape uses is written). The buffer is one static device array
+ * of 2 * 4096 ints (32 KB) per GPU, held until the process ends; its address
+ * is looked up once per GPU, on the first call made with that GPU current
+ * (make that call outside a graph capture). Limits: world_size <= 64,
+ * num_local_experts <= 64 (so num_experts <= 4096): MOE_A2A_ESCRATCH beyond,
+ * before anything is launched.
+ * All calls on one GPU share the buffer, which keeps what the last call wrote:
+ * a second call overwrites the plan of the first, so finish (or at least
+ * enqueue on the same stream) the moe_a2a_combine_send that uses a plan before
+ * the next moe_a2a_dispatch_recv_static on that GPU. Calls that overlap on one
+ * GPU on different streams race.
+ */
+int moe_a2a_dispatch_recv_static(const moe_a2a_shape* shape, const void* recv_buf,
+                                 const int32_t* recv_meta, const int32_t* recv_counts,
+                                 int32_t rows_hint, int32_t capacity_rows,
+                                 int32_t* expert_num_tokens, void* expert_x,
+                                 int32_t* expert_meta, const int32_t** send_back_plan,
+                                 void* stream);
 
 /*
  * Combine, send side: expert-major results -> rows grouped by origin rank.

@@ -95,6 +95,16 @@ def test_bad_arguments_are_rejected_without_touching_the_gpu():
     assert lib.moe_a2a_dispatch_recv(C.byref(ok), one, one, one, 4, -1, one, one, one, None, None) == -1
     assert lib.moe_a2a_dispatch_recv(C.byref(ok), one, one, one, 4, 1 << 30, one, one, one, None, None) == -1
     assert lib.moe_a2a_dispatch_recv(C.byref(ok), None, one, one, 0, 4, one, one, one, None, None) == -1
+    where = C.c_void_p(123)
+    assert lib.moe_a2a_dispatch_recv_static(C.byref(ok), one, one, one, 4, 4, one, one, one, None, None) == -1
+    assert lib.moe_a2a_dispatch_recv_static(None, one, one, one, 4, 4, one, one, one, C.byref(where), None) == -1
+    # beyond the static buffer: more than 64 local experts, more than 64 ranks
+    for big in (_lib.Shape(8, 0, 8 * 65, 8, 64, 16), _lib.Shape(128, 0, 128, 2, 64, 16)):
+        where.value = 123
+        assert lib.moe_a2a_dispatch_recv_static(C.byref(big), one, one, one, 4, 4, one, one, one,
+                                                C.byref(where), None) == -4
+        assert where.value is None  # no plan address is handed out with an error
+    assert b"static buffer" in lib.moe_a2a_strerror(-4)
     assert lib.moe_a2a_combine_send(C.byref(ok), one, one, one, -1, 4, one, one, one, None, None) == -1
     assert lib.moe_a2a_combine_send(C.byref(ok), one, one, one, 4, -1, one, one, one, None, None) == -1
     assert lib.moe_a2a_combine_send(C.byref(ok), one, one, one, 4, 4, None, one, one, None, None) == -1
@@ -173,7 +183,9 @@ def test_torch_extension_wraps_every_entry_point():
     m = _ext.load()
     assert m.a2a_version() == _lib.load().moe_a2a_version().decode()
     wrapped = {"moe_" + f for f in EXT_FUNCTIONS}
-    assert wrapped == set(declared_functions()) - {"moe_a2a_strerror"}
+    # not wrapped: the message lookup, and the variant for callers that cannot allocate (it hands
+    # back a raw device address, which has no torch::Tensor form)
+    assert wrapped == set(declared_functions()) - {"moe_a2a_strerror", "moe_a2a_dispatch_recv_static"}
     source = (ROOT / "amd_distributed_2025_amd" / "csrc" / "moe_a2a_torch.cpp").read_text()
     for f in EXT_FUNCTIONS:
         assert hasattr(m, f), f
