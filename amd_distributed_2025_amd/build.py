@@ -52,9 +52,19 @@ def hipcc_path() -> str:
     raise RuntimeError("hipcc not found (looked at $HIPCC, PATH and /opt/rocm/bin)")
 
 
+def source_id() -> str:
+    """What `moe_a2a_build_id()` of a library built from the present sources returns."""
+    import hashlib
+
+    h = hashlib.sha256(SOURCE.read_bytes())
+    h.update((REPO_DIR / "include" / "moe_a2a.h").read_bytes())
+    return h.hexdigest()[:16]
+
+
 def build_library(verbose: bool = False) -> Path:
     """Compile unconditionally and return the path of the shared library."""
-    cmd = [hipcc_path(), *HIPCC_FLAGS, f"-I{REPO_DIR / 'include'}", str(SOURCE), "-o", str(LIBRARY)]
+    cmd = [hipcc_path(), *HIPCC_FLAGS, f'-DMOE_A2A_BUILD_ID="{source_id()}"', f"-I{REPO_DIR / 'include'}",
+           str(SOURCE), "-o", str(LIBRARY)]
     if verbose:
         print(" ".join(cmd), flush=True)
     proc = subprocess.run(cmd, capture_output=True, text=True)

@@ -69,6 +69,12 @@ typedef struct moe_a2a_shape {
  * "moe_a2a 0.4 gfx950"; the number changes with the ABI. Never NULL. */
 const char* moe_a2a_version(void);
 
+/* Identifies the sources this library was built from: the first 16 hex digits of
+ * the SHA-256 of the kernel source followed by this header, as the build step
+ * computed it, or "unknown" for a build that did not pass it. Measurements kept
+ * on file name the build they were taken on with it. Never NULL. */
+const char* moe_a2a_build_id(void);
+
 /* Human-readable text for a status code. Never NULL. */
 const char* moe_a2a_strerror(int status);
 

@@ -30,6 +30,9 @@ def test_library_exports_every_declared_symbol():
     bound = set(_lib.SIGNATURES) | set(_lib.STRING_FUNCTIONS)
     assert bound == set(declared_functions())
     assert lib.moe_a2a_version().decode().startswith("moe_a2a")
+    # the library on disk was built from the sources on disk
+    from amd_distributed_2025_amd.build import source_id
+    assert lib.moe_a2a_build_id().decode() == source_id()
 
 
 def test_argument_counts_match_the_header():
@@ -185,7 +188,8 @@ def test_torch_extension_wraps_every_entry_point():
     wrapped = {"moe_" + f for f in EXT_FUNCTIONS}
     # not wrapped: the message lookup, and the variant for callers that cannot allocate (it hands
     # back a raw device address, which has no torch::Tensor form)
-    assert wrapped == set(declared_functions()) - {"moe_a2a_strerror", "moe_a2a_dispatch_recv_static"}
+    assert wrapped == set(declared_functions()) - {"moe_a2a_strerror", "moe_a2a_build_id",
+                                                   "moe_a2a_dispatch_recv_static"}
     source = (ROOT / "amd_distributed_2025_amd" / "csrc" / "moe_a2a_torch.cpp").read_text()
     for f in EXT_FUNCTIONS:
         assert hasattr(m, f), f
