@@ -526,8 +526,8 @@ __global__ __launch_bounds__(BLOCK) void dispatch_fanout_kernel(
 }
 
 // The same fan-out for rows longer than 256 vectors: a workgroup of BLK = 512
-// lanes holds one vector per lane, so a row is cut into half as many chunks and
-// its K entries are ranked half as often. A lane compares 2048 / BLK keys per
+// lanes holds NV vectors per lane (BLK lanes apart), so a row is cut into fewer
+// chunks and its K entries are ranked less often. A lane compares 2048 / BLK keys per
 // batch; the per-wave counts travel as 16-bit pairs (entry g with entry g + 4),
 // are summed across the waves by the DPP row scan of one wave (a row of 16
 // lanes per pair) and come back through LDS. Needs S < 65536 for the pairs not
@@ -536,7 +536,7 @@ __global__ __launch_bounds__(BLOCK) void dispatch_fanout_kernel(
 // the whole step 0.3 us shorter than with 256 lanes; 1024 lanes (one chunk per
 // row) 0.5 us longer.
 
-template <typename V, int BLK, bool POW2>
+template <typename V, int BLK, int NV, bool POW2>
 __global__ __launch_bounds__(BLK) void dispatch_fanout_wide_kernel(
     const V* __restrict__ x, const int* __restrict__ indices, int T, int K, int nle, int E, int W,
     uint32_t magic, int nle_shift, int order_bits, int rank, int row_vecs, int chunks,
@@ -570,13 +570,15 @@ __global__ __launch_bounds__(BLK) void dispatch_fanout_wide_kernel(
   const int items = T * chunks, movers = gridDim.x - W;
   for (int q = blockIdx.x - W; q < items; q += movers) {
     const int t = chunks == 1 ? q : q / chunks, c = q - t * chunks;
-    const int col = c * BLK + tid;
+    const int col = c * (BLK * NV) + tid;  // this lane's first vector; the others BLK apart
     const int i0 = t * K;
 
     int key[KEYS];
 #pragma unroll
     for (int u = 0; u < KEYS; ++u) key[u] = indices[min(tid + u * BLK, S - 1)];
-    const V v = stream_load(x + (size_t)t * row_vecs + min(col, row_vecs - 1));
+    V v[NV];
+#pragma unroll
+    for (int j = 0; j < NV; ++j) v[j] = stream_load(x + (size_t)t * row_vecs + min(col + j * BLK, row_vecs - 1));
 
     for (int g0 = 0; g0 < K; g0 += FAN) {
       int mine[FAN];
@@ -633,8 +635,10 @@ __global__ __launch_bounds__(BLK) void dispatch_fanout_wide_kernel(
       const int live = min(FAN, K - g0);
 #pragma unroll
       for (int g = 0; g < FAN; ++g) {
-        if (g < live && col < row_vecs)
-          row_store<(MOE_A2A_NT_SEND != 0)>(send_buf + (size_t)slot[g] * row_vecs + col, v);
+#pragma unroll
+        for (int j = 0; j < NV; ++j)
+          if (g < live && col + j * BLK < row_vecs)
+            row_store<(MOE_A2A_NT_SEND != 0)>(send_buf + (size_t)slot[g] * row_vecs + col + j * BLK, v[j]);
       }
       if (c == 0 && tid < live * META) {
         const int g = tid / META, f = tid - g * META;
@@ -1749,20 +1753,30 @@ int moe_a2a_dispatch_send(const moe_a2a_shape* s, const void* x, const int32_t* 
 #endif
     constexpr int WIDE = 2 * BLOCK;  // rows of more than one 256-lane chunk: 512-lane workgroups
     if (MOE_A2A_FANOUT_WIDE && f.row_vecs > BLOCK && S < 65536 && s->world_size < 16384) {
-      const int wchunks = (f.row_vecs + WIDE - 1) / WIDE;
+      // Rows of more than 512 vectors: two vectors per lane, so that a row of up to 1024 vectors
+      // is one workgroup's and its entries are ranked once, not once per chunk (measured at
+      // H = 7168: the whole step 0.4 us shorter; 256 lanes x 4 and 1024 lanes x 1 were slower).
+      const int fnv = f.row_vecs > WIDE ? 2 : 1;
+      const int wchunks = (f.row_vecs + WIDE * fnv - 1) / (WIDE * fnv);
       const int wgrid = s->world_size + mover_blocks((long long)num_tokens * wchunks);
       int order_bits = 1;  // S <= 1 << order_bits <= 65536, so (W + 1) << order_bits fits an int
       while ((1ll << order_bits) < S) ++order_bits;
       const bool pow2 = (g.nle & (g.nle - 1)) == 0;
       int nle_shift = 0;
       while ((1 << nle_shift) < g.nle) ++nle_shift;
-#define LAUNCH_W(V, POW2)                                                                      \
-  dispatch_fanout_wide_kernel<V, WIDE, POW2><<<wgrid, WIDE, 0, st>>>(                          \
+#define LAUNCH_W(V, NV, POW2)                                                                  \
+  dispatch_fanout_wide_kernel<V, WIDE, NV, POW2><<<wgrid, WIDE, 0, st>>>(                      \
       (const V*)x, indices, num_tokens, s->experts_per_token, g.nle, s->num_experts,           \
       s->world_size, g.magic, nle_shift, order_bits, s->rank, f.row_vecs, wchunks,             \
       (V*)send_buf, send_meta, send_counts, send_slot)
-      if (f.vec16) { if (pow2) LAUNCH_W(b128, true); else LAUNCH_W(b128, false); }
-      else { if (pow2) LAUNCH_W(uint16_t, true); else LAUNCH_W(uint16_t, false); }
+#define LAUNCH_WV(V)                                                  \
+  do {                                                                \
+    if (fnv == 2) { if (pow2) LAUNCH_W(V, 2, true); else LAUNCH_W(V, 2, false); } \
+    else { if (pow2) LAUNCH_W(V, 1, true); else LAUNCH_W(V, 1, false); }          \
+  } while (0)
+      if (f.vec16) LAUNCH_WV(b128);
+      else LAUNCH_WV(uint16_t);
+#undef LAUNCH_WV
 #undef LAUNCH_W
       return launch_status();
     }

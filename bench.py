@@ -15,11 +15,14 @@ kernels on their seeded inputs; they stay resident where an exchange would have 
 
 Prints ONE JSON line. `value` is the wall time of a whole step (stand-ins included) in microseconds, the
 mean over exactly `--steps` graph replays between two synchronisations; `step_us_median` / `step_us_min`
-are taken over batches of the same replays timed with events. `hot_path_us` is the sum of the four path
-kernels, each timed in place (HIP events on the launch stream around graphs of whole steps with and
-without that kernel); `roofline` prices the slowest of those four against HBM peak with the algorithmic
-bytes of its stage; `ranks` repeats the hot-path figure for every rank of the job (their received row
-counts differ); `cpu_baseline` is the row-by-row torch-CPU statement of the same step timed on this box's
+are taken over batches of the same replays timed with events. `hot_path_us` is the time of the four path
+launches by themselves: HIP events on the launch stream around a graph that holds `--kernel-reps` times
+dispatch_send, dispatch_recv, combine_send, combine_recv and nothing else, every input resident where
+the step leaves it. The cost of one of them is that time minus the time of the same graph without it;
+`roofline` prices the slowest against HBM peak with the algorithmic bytes of its stage.
+`hot_path_us_in_step` is the whole step minus a step of the three stand-ins alone. `ranks` repeats the
+hot-path figure for every rank of the job (their received row counts differ); `cpu_baseline` is the
+row-by-row torch-CPU statement of the same step timed on this box's
 host cores, with the vectorised numpy statement beside it; `custom_kernel_wall_us` is one call of the
 reference's entry point (which steps all ranks of the job on this one GPU).
 """
@@ -55,7 +58,7 @@ def parse_args():
     ap.add_argument("--mode", default="graph", choices=["graph", "eager"],
                     help="replay a captured HIP graph of the step (default) or launch eagerly")
     ap.add_argument("--kernel-reps", type=int, default=20,
-                    help="whole steps per graph in the per-kernel (leave-one-out) timing")
+                    help="repetitions of the launches inside each timing graph")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="target CPU time of the cpu_baseline sample")
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
     ap.add_argument("--no-rank-sweep", action="store_true", help="time only --rank, not every rank of the job")
@@ -176,29 +179,31 @@ def main():
             samples.append(e0.elapsed_time(e1) * 1e3 / reps)
         return statistics.median(samples)
 
-    # Per-kernel cost in the pipeline: HIP events on the launch stream around a graph of `reps` whole
-    # steps, with and without the kernel. The difference is what the kernel costs where it runs, with
-    # its inputs in the cache state the previous kernel left them in (its launch gap included). A
-    # kernel timed alone in a loop re-reads inputs that nothing rewrote and looks faster.
-    def kernel_costs(stages, T, R, alone=False):
+    # The path by itself: a graph of `reps` times the four path launches, timed with HIP events on the
+    # launch stream. A kernel's cost is what the graph loses when the kernel is left out. (Leaving a
+    # kernel out of the WHOLE step does not give a usable figure: with the small exchange stand-ins in
+    # the graph the parts add up to between 3 us less and 1 us more than the whole, and the sum moves
+    # by microseconds between builds whose whole step differs by half a microsecond.)
+    def path_costs(stages, T, R, per_kernel=True, alone=False):
         reps = args.kernel_reps
-        full_us = time_graph(graph_of([fn for _, fn in stages], reps), reps)
+        path = [(n, f) for n, f in stages if n in PATH]
+        chain_us = time_graph(graph_of([f for _, f in path], reps), reps)
         kern = {}
-        for name, fn in stages:
-            without = time_graph(graph_of([f for n, f in stages if n != name], reps), reps)
-            kern[name] = {"us": round(full_us - without, 3)}
-            if alone:  # the kernel back to back with itself: inputs stay warm, no producer in between
-                kern[name]["us_alone_warm"] = round(time_graph(graph_of([fn], reps), reps), 3)
+        if per_kernel:
+            for name, fn in path:
+                without = time_graph(graph_of([f for n, f in path if n != name], reps), reps)
+                kern[name] = {"us": round(chain_us - without, 3)}
+                if alone:  # the kernel back to back with itself: inputs stay warm, no producer in between
+                    kern[name]["us_alone_warm"] = round(time_graph(graph_of([fn], reps), reps), 3)
+            ab = alg_bytes(T, K, H, R)
+            for name in PATH:
+                kern[name]["alg_bytes"] = ab[name]
+                kern[name]["gbps"] = round(ab[name] / kern[name]["us"] * 1e-3, 1)
+                kern[name]["frac"] = round(kern[name]["gbps"] / HBM_PEAK_GBPS, 4)
         for _, fn in stages:  # leave every buffer as a full step leaves it
             fn()
         torch.cuda.synchronize()
-        ab = alg_bytes(T, K, H, R)
-        for name in PATH:
-            kern[name]["alg_bytes"] = ab[name]
-            kern[name]["gbps"] = round(ab[name] / kern[name]["us"] * 1e-3, 1)
-            kern[name]["frac"] = round(kern[name]["gbps"] / HBM_PEAK_GBPS, 4)
-        hot_us = sum(kern[n]["us"] for n in PATH)
-        return full_us, kern, hot_us, sum(ab.values())
+        return chain_us, kern, sum(alg_bytes(T, K, H, R).values())
 
     r0 = args.rank
     stages, T, R, y = stages_of(r0)
@@ -236,7 +241,10 @@ def main():
         e1.synchronize()
         batches.append(e0.elapsed_time(e1) * 1e3 / batch)
 
-    full_us, kern, hot_us, total_alg = kernel_costs(stages, T, R, alone=args.alone)
+    hot_us, kern, total_alg = path_costs(stages, T, R, alone=args.alone)
+    reps = args.kernel_reps
+    full_us = time_graph(graph_of([fn for _, fn in stages], reps), reps)
+    standins_us = time_graph(graph_of([fn for n, fn in stages if n not in PATH], reps), reps)
     dominant = max(PATH, key=lambda n: kern[n]["us"])
     build_id = lib.moe_a2a_build_id().decode()
 
@@ -264,6 +272,9 @@ def main():
         "step_us_min": round(min(batches), 3),
         "step_us_graph_of_steps": round(full_us, 3),
         "hot_path_us": round(hot_us, 3),
+        "hot_path_measure": f"graph of {reps} x the four path launches, HIP events, median of 9",
+        "hot_path_us_in_step": round(full_us - standins_us, 3),
+        "hot_path_kernel_sum_us": round(sum(kern[n]["us"] for n in PATH), 3),
         "hot_path_alg_bytes": total_alg,
         "hot_path_gbps": round(total_alg / hot_us * 1e-3, 1),
         "hot_path_frac_of_hbm_peak": round(total_alg / hot_us * 1e-3 / HBM_PEAK_GBPS, 4),
@@ -286,7 +297,7 @@ def main():
                 hot_r, alg_r, rows_r = hot_us, total_alg, R
             else:
                 st_r, T_r, R_r, _ = stages_of(r)
-                _, _, hot_r, alg_r = kernel_costs(st_r, T_r, R_r)
+                hot_r, _, alg_r = path_costs(st_r, T_r, R_r, per_kernel=False)
                 rows_r = R_r
             ranks[str(r)] = {"rows_received": rows_r, "hot_path_us": round(hot_r, 3),
                              "frac": round(alg_r / hot_r * 1e-3 / HBM_PEAK_GBPS, 4)}

@@ -153,6 +153,11 @@ EDGE = {
                                       max_num_tokens=6, num_tokens="full", dtype="fp16"),
     "wide_fanout_twelve_entries": dict(world_size=2, num_experts=24, experts_per_token=12, hidden_dim=4104,
                                        max_num_tokens=9, num_tokens="uniform", dtype="bf16"),
+    "wide_fanout_two_vectors_per_lane_two_chunks": dict(world_size=2, num_experts=8, experts_per_token=4,
+                                                        hidden_dim=8200, max_num_tokens=7, num_tokens="full",
+                                                        dtype="bf16"),
+    "wide_fanout_odd_local_experts": dict(world_size=4, num_experts=12, experts_per_token=5, hidden_dim=7168,
+                                          max_num_tokens=11, num_tokens="uniform", dtype="fp16"),
     "k_above_fast_list": dict(world_size=2, num_experts=160, experts_per_token=72, hidden_dim=64,
                               max_num_tokens=3, num_tokens="full", dtype="bf16"),
 }
