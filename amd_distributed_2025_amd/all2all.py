@@ -167,6 +167,25 @@ class HIPAllToAll:
         self.binding.expert_scale(self.shape, expert_x, expert_num_tokens, hint, ey, _stream(self.device))
         return ey
 
+    def expert_gemm(self, expert_x, expert_num_tokens, weights, rows_hint: Optional[int] = None):
+        """The expert computation as a grouped GEMM: `expert_x[le, j] @ weights[le].T` on the valid
+        rows, float32 accumulation, one rounding. `weights` is [nle, H, H] of the row type with the
+        input index contiguous. Takes the place of all2all/reference.py:262 in a model; needs
+        in_dtype == out_dtype and hidden_dim % 64 == 0."""
+        cfg = self.cfg
+        if cfg.in_dtype != cfg.out_dtype:
+            raise ValueError("expert_gemm computes in one 16-bit type: in_dtype must equal out_dtype")
+        nle = cfg.num_experts // self.world_size
+        _need(expert_x, cfg.in_dtype, self.device, "expert_x")
+        _need(expert_num_tokens, torch.int32, self.device, "expert_num_tokens")
+        _need(weights, cfg.in_dtype, self.device, "weights")
+        if tuple(weights.shape) != (nle, cfg.hidden_dim, cfg.hidden_dim):
+            raise ValueError(f"weights must be [{nle}, {cfg.hidden_dim}, {cfg.hidden_dim}], got {tuple(weights.shape)}")
+        hint = self._default_rows_in(rows_hint)
+        ey = self._buf("expert_y", tuple(expert_x.shape), cfg.out_dtype)
+        self.binding.expert_gemm(self.shape, expert_x, expert_num_tokens, hint, weights, ey, _stream(self.device))
+        return ey
+
     def combine_send(self, expert_meta, expert_y, expert_num_tokens, rows_hint: Optional[int] = None):
         """Expert-major results -> rows grouped by origin rank.
         Returns (back_counts int32[W], back_buf [max_rows_in,H], back_meta [max_rows_in,5]);

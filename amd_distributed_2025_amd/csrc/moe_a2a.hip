@@ -922,17 +922,16 @@ __global__ __launch_bounds__(64 * ROWS) void dispatch_recv_kernel(
 
 // ---------------------------------------------------------------- expert-major stream helpers
 
-// pre[0..nle] = exclusive prefix of min(cnt[le], max_recv); returns the total.
-// Each lane owns a contiguous run of experts; runs are combined by a wave64
-// scan and a scan over the wave totals.
-template <int NW>
-__device__ __forceinline__ int expert_prefix(const int* __restrict__ cnt, int nle, int max_recv,
-                                             int* pre, int* red) {
+// pre[0..nle] = exclusive prefix of value_of(le); returns the total. Each lane
+// owns a contiguous run of experts; runs are combined by a wave64 scan and a
+// scan over the wave totals.
+template <int NW, class ValueOf>
+__device__ __forceinline__ int expert_prefix_of(int nle, int* pre, int* red, ValueOf value_of) {
   const int tid = threadIdx.x;
   const int per = (nle + 64 * NW - 1) / (64 * NW);
   const int b = min(tid * per, nle), e = min(b + per, nle);
   int s = 0;
-  for (int i = b; i < e; ++i) s += min(max(cnt[i], 0), max_recv);
+  for (int i = b; i < e; ++i) s += value_of(i);
   const int inc = wave_inclusive_scan(s);
   if ((tid & 63) == 63) red[tid >> 6] = inc;
   lds_barrier();
@@ -945,11 +944,18 @@ __device__ __forceinline__ int expert_prefix(const int* __restrict__ cnt, int nl
   int run = off + inc - s;
   for (int i = b; i < e; ++i) {
     pre[i] = run;
-    run += min(max(cnt[i], 0), max_recv);
+    run += value_of(i);
   }
   if (tid == 0) pre[nle] = total;
   lds_barrier();
   return total;
+}
+
+// The prefix of the rows per expert, min(cnt[le], max_recv).
+template <int NW>
+__device__ __forceinline__ int expert_prefix(const int* __restrict__ cnt, int nle, int max_recv,
+                                             int* pre, int* red) {
+  return expert_prefix_of<NW>(nle, pre, red, [=](int le) { return min(max(cnt[le], 0), max_recv); });
 }
 
 // Largest le in [0, nle) with pre[le] <= g, for g < pre[nle] (so empty experts
@@ -1544,6 +1550,133 @@ __global__ __launch_bounds__(64 * ROWS) void expert_scale_wave_kernel(
   }
 }
 
+// ---------------------------------------------------------------- expert computation: grouped GEMM
+//
+// expert_y[le, j, :] = expert_x[le, j, :] @ W[le]^T for the valid rows j < expert_num_tokens[le] of
+// the padded expert-major buffers: what stands where all2all/reference.py:262 has the simulated
+// expert. W[le] is [H_out = H, H_in = H] with the input index contiguous (the layout of a linear
+// layer's weight), so that both MFMA operands are read straight from memory in the layout
+// v_mfma_f32_32x32x16 wants: a lane holds 8 consecutive input elements of one row.
+//
+// With a few dozen rows per expert the problem is bound by streaming the weights (at C4: 3.3 GB of
+// them for 0.2 PFLOP), so the kernel is built to keep weight bytes in flight, not to keep the MFMA
+// pipe full. A workgroup of 4 waves owns a tile of 128 tokens x 128 output columns of one expert,
+// a wave 64 x 64 of it (2 x 2 MFMA tiles, fp32 accumulators in registers), and walks the input
+// dimension 64 elements at a time with the next step's operands requested before the current
+// step's 16 MFMAs are issued. Operands go from global memory to registers: a weight element is used
+// by one workgroup only (an expert with at most 128 rows has one tile of tokens), and the token rows
+// of a tile are re-read by the workgroups of the other column tiles from the L2. No LDS, no barrier
+// in the main loop. The MFMA computes the tile transposed (weights as the A operand, tokens as B),
+// which leaves a lane holding four consecutive output columns of one token: 8-byte stores.
+//
+// Tiles are numbered over (expert, 128-row block) by a prefix over the device-side counts, so a hot
+// expert is spread over as many workgroups as it has blocks of rows and an empty one costs nothing.
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+
+template <int DT> struct Mfma32x32x16;
+template <> struct Mfma32x32x16<MOE_A2A_BF16> {
+  static __device__ __forceinline__ f32x16 mma(b128 a, b128 b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+  }
+};
+template <> struct Mfma32x32x16<MOE_A2A_F16> {
+  static __device__ __forceinline__ f32x16 mma(b128 a, b128 b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+  }
+};
+
+constexpr int GEMM_TILE = 128;   // tokens and output columns per workgroup
+constexpr int GEMM_WAVE = 64;    // tokens and output columns per wave
+constexpr int GEMM_KSTEP = 64;   // input elements per step: a lane reads 64 contiguous bytes of a row
+
+template <int DT>
+__global__ __launch_bounds__(BLOCK, 2) void expert_gemm_kernel(
+    const b128* __restrict__ expert_x, const int* __restrict__ expert_num_tokens,
+    const b128* __restrict__ weights, uint16_t* __restrict__ expert_y, int nle, int max_recv, int H,
+    int col_tiles) {
+  __shared__ int red[NWAVES];
+  __shared__ int pre[MAX_LOCAL_EXPERTS + 1];  // row blocks before each expert
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  expert_prefix_of<NWAVES>(nle, pre, red, [=](int le) {  // blocks of 128 rows per expert
+    return (min(max(expert_num_tokens[le], 0), max_recv) + GEMM_TILE - 1) / GEMM_TILE;
+  });
+  const int row_blocks = pre[nle];
+  const int top = top_step(nle);
+  const int row_vecs = H / 8;                 // 16-byte vectors per row
+  const int wm = wave & 1, wn = wave >> 1;    // this wave's quarter of the tile
+  const int r = lane & 31, kb = lane >> 5;    // MFMA operand layout: row r, input elements kb*8 .. kb*8+7 of a 16-block
+
+  const int tiles = row_blocks * col_tiles, stride = gridDim.x;
+  for (int tile = blockIdx.x; tile < tiles; tile += stride) {
+    const int rb = tile / col_tiles, ct = tile - rb * col_tiles;
+    const int le = expert_of(pre, nle, top, rb);
+    const int rows = min(max(expert_num_tokens[le], 0), max_recv);
+    const int m0 = (rb - pre[le]) * GEMM_TILE + wm * GEMM_WAVE;  // first token of this wave
+    const int n0 = ct * GEMM_TILE + wn * GEMM_WAVE;              // first output column of this wave
+    if (m0 >= rows || n0 >= H) continue;  // (no barrier below: a wave may skip its quarter)
+
+    // rows of the two operands this lane reads: output columns n0 + i*32 + r of W, tokens m0 + j*32 + r of x
+    const b128* wrow[2];
+    const b128* xrow[2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      wrow[i] = weights + ((size_t)le * H + n0 + i * 32 + r) * row_vecs + kb * 4;
+      xrow[i] = expert_x + ((size_t)le * max_recv + min(m0 + i * 32 + r, rows - 1)) * row_vecs + kb * 4;
+    }
+    f32x16 acc[2][2] = {};
+    b128 wv[2][4], xv[2][4];
+    auto fetch = [&](b128 (&wreg)[2][4], b128 (&xreg)[2][4], int k8) {  // k8: step offset in vectors
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          wreg[i][q] = wrow[i][k8 + q];
+          xreg[i][q] = xrow[i][k8 + q];
+        }
+    };
+    fetch(wv, xv, 0);
+    for (int k8 = 0; k8 < row_vecs; k8 += GEMM_KSTEP / 8) {
+      b128 wn_[2][4], xn_[2][4];
+      const int next = min(k8 + GEMM_KSTEP / 8, row_vecs - GEMM_KSTEP / 8);  // the last step re-reads itself
+      fetch(wn_, xn_, next);
+#pragma unroll
+      for (int q = 0; q < 4; ++q)
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+#pragma unroll
+          for (int j = 0; j < 2; ++j) acc[i][j] = Mfma32x32x16<DT>::mma(wv[i][q], xv[j][q], acc[i][j]);
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          wv[i][q] = wn_[i][q];
+          xv[i][q] = xn_[i][q];
+        }
+    }
+    // D[n][m] of a 32x32 tile: this lane holds token m = r and output columns (g*8 + kb*4 + 0..3), g < 4
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int token = m0 + j * 32 + r;
+      if (token < rows) {
+        uint16_t* out = expert_y + ((size_t)le * max_recv + token) * H + n0 + kb * 4;
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+#pragma unroll
+          for (int g = 0; g < 4; ++g) {
+            const f32x16& a = acc[i][j];
+            uint32_t two[2] = {Pair16<DT>::round(a[g * 4 + 0], a[g * 4 + 1]), Pair16<DT>::round(a[g * 4 + 2], a[g * 4 + 3])};
+            two[0] = Pair16<DT>::canonical(two[0]);
+            two[1] = Pair16<DT>::canonical(two[1]);
+            __builtin_memcpy(out + i * 32 + g * 8, two, 8);
+          }
+      }
+    }
+  }
+}
+
 // ---------------------------------------------------------------- exchange stand-in
 
 template <typename V, int NV>
@@ -2023,6 +2156,33 @@ int moe_a2a_expert_scale(const moe_a2a_shape* s, const void* expert_x,
   MOE_A2A_FOR_ROW_KERNEL(g, LAUNCH);
 #undef LAUNCH
 #undef LAUNCH_T
+  return launch_status();
+}
+
+int moe_a2a_expert_gemm(const moe_a2a_shape* s, const void* expert_x,
+                        const int32_t* expert_num_tokens, int32_t rows_hint, const void* weights,
+                        int32_t dtype, void* expert_y, void* stream) {
+  if (!shape_ok(s) || rows_hint < 0 || !expert_x || !expert_num_tokens || !weights || !expert_y)
+    return MOE_A2A_EINVAL;
+  if (dtype != MOE_A2A_F16 && dtype != MOE_A2A_BF16) return MOE_A2A_EINVAL;
+  if (s->hidden_dim % GEMM_KSTEP != 0) return MOE_A2A_EINVAL;  // whole steps of the input, whole wave tiles of columns
+  if (!all_aligned(16, expert_x, weights, expert_y)) return MOE_A2A_EALIGN;
+  const int nle = s->num_experts / s->world_size;
+  if (nle > MAX_LOCAL_EXPERTS) return MOE_A2A_EINVAL;
+  const long long max_recv = (long long)s->max_num_tokens * s->world_size;
+  const int col_tiles = (s->hidden_dim + GEMM_TILE - 1) / GEMM_TILE;
+  // every expert can end in a partly filled block of rows; the kernel strides over what the hint misses
+  const long long row_blocks = (long long)rows_hint / GEMM_TILE + nle;
+  if ((max_recv / GEMM_TILE + 1) * nle * col_tiles > INT_MAX / 2) return MOE_A2A_EINVAL;
+  const int grid = mover_blocks(row_blocks * col_tiles);
+  hipStream_t st = (hipStream_t)stream;
+#define LAUNCH_G(DT)                                                                         \
+  expert_gemm_kernel<DT><<<grid, BLOCK, 0, st>>>((const b128*)expert_x, expert_num_tokens,   \
+                                                 (const b128*)weights, (uint16_t*)expert_y,  \
+                                                 nle, (int)max_recv, s->hidden_dim, col_tiles)
+  if (dtype == MOE_A2A_BF16) LAUNCH_G(MOE_A2A_BF16);
+  else LAUNCH_G(MOE_A2A_F16);
+#undef LAUNCH_G
   return launch_status();
 }
 

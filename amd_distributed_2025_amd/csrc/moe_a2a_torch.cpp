@@ -184,6 +184,21 @@ void a2a_expert_scale(std::vector<int64_t> shape, torch::Tensor expert_x, torch:
          "moe_a2a_expert_scale");
 }
 
+void a2a_expert_gemm(std::vector<int64_t> shape, torch::Tensor expert_x, torch::Tensor expert_num_tokens,
+                     int64_t rows_hint, torch::Tensor weights, torch::Tensor expert_y, int64_t stream) {
+  const moe_a2a_shape s = shape_of(shape);
+  const auto dt = rows_type(expert_x, "expert_x");
+  const int64_t nle = s.world_size > 0 ? s.num_experts / s.world_size : 0;
+  const int64_t padded = nle * s.max_num_tokens * s.world_size;
+  need(expert_x, "expert_x", dt, padded * s.hidden_dim);
+  need(expert_y, "expert_y", dt, padded * s.hidden_dim, &expert_x);
+  need(weights, "weights", dt, nle * s.hidden_dim * s.hidden_dim, &expert_x);
+  need(expert_num_tokens, "expert_num_tokens", torch::kInt32, nle, &expert_x);
+  status(moe_a2a_expert_gemm(&s, expert_x.data_ptr(), ints(expert_num_tokens), to_i32(rows_hint, "rows_hint"),
+                             weights.data_ptr(), dtype_code(dt), expert_y.data_ptr(), stream_of(stream)),
+         "moe_a2a_expert_gemm");
+}
+
 void a2a_exchange_local(int64_t world_size, int64_t hidden_dim, torch::Tensor send_buf, torch::Tensor send_meta,
                         torch::Tensor send_counts, int64_t dst_rank, torch::Tensor recv_buf,
                         torch::Tensor recv_meta, torch::Tensor recv_counts, int64_t src_rank, int64_t rows_hint,

@@ -256,6 +256,39 @@ int moe_a2a_expert_scale(const moe_a2a_shape* shape, const void* expert_x,
                          void* stream);
 
 /*
+ * The expert computation between dispatch and combine as a grouped GEMM over the
+ * expert-major layout: for every local expert le and every valid row
+ * j < expert_num_tokens[le]
+ *   expert_y[le, j, :] = expert_x[le, j, :] @ weights[le]^T
+ * with float32 accumulation and one rounding to the 16-bit type. It fills the
+ * place of all2all/reference.py:262, where the reference has the simulated
+ * expert `expert_x.to(out_dtype) * (1 + rank)` (moe_a2a_expert_scale keeps that
+ * arithmetic for parity with the reference; this is what a model would run
+ * there).
+ *
+ *   expert_x   [nle, max_recv, H], expert_num_tokens [nle] as moe_a2a_dispatch_recv
+ *              leaves them (counts above max_recv are clamped)
+ *   weights    [nle, H, H] of the same 16-bit type: weights[le][n][k] multiplies
+ *              input element k into output element n (the layout of a linear
+ *              layer's weight, input index contiguous)
+ *   dtype      MOE_A2A_F16 or MOE_A2A_BF16: element type of all three
+ *   expert_y   [nle, max_recv, H] out; rows at or past expert_num_tokens[le] are
+ *              not written
+ * Rows are processed in blocks of 128 found from the device-side counts, so the
+ * work follows the rows, not the experts. Limits: hidden_dim a multiple of 64,
+ * all three buffers 16-byte aligned, nle <= 4096 (MOE_A2A_EINVAL / EALIGN).
+ * Sums are formed in float32 in the order of the matrix unit, which is not the
+ * order of a CPU matmul: results agree with a float32 reference to within one
+ * unit in the last place of the 16-bit type plus the float32 summation error,
+ * and exactly when every sum has at most one nonzero term per 16 inputs that is
+ * exactly representable (identity and signed permutation weights).
+ */
+int moe_a2a_expert_gemm(const moe_a2a_shape* shape, const void* expert_x,
+                        const int32_t* expert_num_tokens, int32_t rows_hint,
+                        const void* weights, int32_t dtype, void* expert_y,
+                        void* stream);
+
+/*
  * Stand-in for one (source rank -> destination rank) leg of the exchange,
  * done as a device copy on one GPU. Replaces, for that leg, the three
  * dist.all_to_all_single calls at all2all/reference.py:107-119 (dispatch)

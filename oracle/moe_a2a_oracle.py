@@ -188,6 +188,32 @@ def expert_scale(rows: np.ndarray, rank: int, in_dtype: str, out_dtype: str) -> 
     return f32_to_b16(as_out * np.float32(1 + rank), out_dtype)
 
 
+def expert_gemm(rows: np.ndarray, weights: np.ndarray, dtype: str) -> np.ndarray:
+    """One expert's rows through a linear layer, `rows @ weights.T`, where a model
+    has its expert and all2all/reference.py:262 has the stand-in: 16-bit operands
+    (`rows` [n, H], `weights` [H_out, H_in] as bit patterns), products and sums in
+    float32, one rounding to the 16-bit type. The order of a float32 sum is not
+    fixed by this statement; `expert_gemm_bound` gives what every order satisfies."""
+    acc = b16_to_f32(rows, dtype) @ b16_to_f32(weights, dtype).T
+    return f32_to_b16(acc.astype(np.float32), dtype)
+
+
+def expert_gemm_bound(rows: np.ndarray, weights: np.ndarray, dtype: str):
+    """(exact, tol): the float64 value of `rows @ weights.T` and the distance from it
+    that a float32-accumulated, once-rounded 16-bit result can have in any summation
+    order: K terms summed in float32 are off by at most K * 2^-24 * sum|x||w|
+    (products of two 16-bit values are exact in float32), and the final rounding
+    by half a unit in the last place (2^-8 relative for bf16, 2^-11 for fp16; the
+    2^-24 / 2^-133 floor covers subnormal results)."""
+    x = b16_to_f32(rows, dtype).astype(np.float64)
+    w = b16_to_f32(weights, dtype).astype(np.float64)
+    exact = x @ w.T
+    mass = np.abs(x) @ np.abs(w).T
+    u16, floor = (2.0 ** -8, 2.0 ** -133) if dtype == "bf16" else (2.0 ** -11, 2.0 ** -24)
+    sum_err = x.shape[1] * 2.0 ** -24 * mass
+    return exact, u16 * (np.abs(exact) + sum_err) + sum_err + floor
+
+
 # ----------------------------------------------------------------------------- combine
 
 

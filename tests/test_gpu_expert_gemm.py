@@ -1,0 +1,192 @@
+"""The grouped GEMM over the expert-major layout (`moe_a2a_expert_gemm`), which a
+model runs where all2all/reference.py:262 has its stand-in expert.
+
+What is exact is tested exactly: weights that are signed permutations, and small
+integers whose sums every summation order represents. Random operands are held to
+the bound that float32 accumulation in any order plus one rounding allows around
+the float64 product (`oracle.expert_gemm_bound`); the float32 oracle is inside the
+same bound, and the two mostly agree to the bit."""
+import numpy as np
+import pytest
+import torch
+
+from amd_distributed_2025_amd import LocalWorld, WORKLOADS
+from amd_distributed_2025_amd.task import MoEConfig, dtype_name
+from oracle import moe_a2a_oracle as orc
+from tests.helpers import bits, from_bits
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+SENTINEL = 0x7B7B  # bit pattern rows past the counts must keep
+
+
+def rank_object(W, nle, H, max_tokens, dt, binding="ctypes"):
+    cfg = MoEConfig(W * nle, 1, H, max_tokens, dt, dt)
+    return LocalWorld(cfg, W, device=DEV, binding=binding).ranks[W - 1], cfg
+
+
+def run_gemm(a, ex, counts, w, hint=None):
+    """Runs the kernel twice into the same buffer, the second time over a buffer of
+    sentinels, and returns the bit patterns of that second result."""
+    num = torch.tensor(counts, dtype=torch.int32, device=DEV)
+    ey = a.expert_gemm(ex, num, w, hint)
+    ey.view(torch.int16).fill_(SENTINEL)
+    again = a.expert_gemm(ex, num, w, hint)
+    assert again.data_ptr() == ey.data_ptr()
+    torch.cuda.synchronize()
+    return bits(again)
+
+
+def check_padding_untouched(got, counts):
+    for le, c in enumerate(counts):
+        assert (got[le, c:] == SENTINEL).all(), f"expert {le}: rows past its {c} were written"
+
+
+def ragged_counts(rng, nle, max_recv, special):
+    counts = rng.integers(0, min(max_recv, 200) + 1, nle)
+    for i, c in enumerate(special):
+        counts[i % nle] = min(c, max_recv)
+    return [int(c) for c in counts]
+
+
+@pytest.mark.parametrize("dt", [torch.bfloat16, torch.float16], ids=["bf16", "fp16"])
+@pytest.mark.parametrize("W,nle,H,max_tokens", [(1, 1, 64, 16), (2, 3, 192, 80), (4, 8, 2048, 128), (8, 2, 7168, 40)])
+def test_signed_permutation_weights_move_columns_exactly(W, nle, H, max_tokens, dt):
+    print(f"permutation W={W} nle={nle} H={H} T={max_tokens} {dt}", flush=True)
+    rng = np.random.default_rng(H + nle)
+    a, cfg = rank_object(W, nle, H, max_tokens, dt)
+    max_recv = W * max_tokens
+    counts = ragged_counts(rng, nle, max_recv, [0, max_recv, 1, 129, 128, 127])
+    xb = rng.integers(0, 1 << 16, (nle, max_recv, H), dtype=np.uint16)
+    name = dtype_name(dt)
+    finite = np.isfinite(orc.b16_to_f32(xb, name))
+    xb[~finite] = 0x3C00
+    perm = np.stack([rng.permutation(H) for _ in range(nle)])
+    sign = rng.choice([-1.0, 1.0], (nle, H))
+    w = torch.zeros(nle, H, H, dtype=dt)
+    for le in range(nle):
+        w[le, torch.arange(H), torch.from_numpy(perm[le])] = torch.from_numpy(sign[le]).to(dt)
+    got = run_gemm(a, from_bits(xb, dt).to(DEV), counts, w.to(DEV))
+    check_padding_untouched(got, counts)
+    for le, c in enumerate(counts):
+        moved = xb[le, :c][:, perm[le]]
+        want = np.where(sign[le] < 0, moved ^ 0x8000, moved).astype(np.uint16)
+        # -0 + 0 sums: a zero's sign is the one thing the order of the sum may change
+        zero = (want & 0x7FFF) == 0
+        assert np.array_equal(got[le, :c][~zero], want[~zero]), f"expert {le}"
+        assert ((got[le, :c][zero] & 0x7FFF) == 0).all()
+
+
+@pytest.mark.parametrize("dt", [torch.bfloat16, torch.float16], ids=["bf16", "fp16"])
+@pytest.mark.parametrize("H", [128, 192])
+def test_small_integers_sum_exactly(H, dt):
+    print(f"integers H={H} {dt}", flush=True)
+    rng = np.random.default_rng(H)
+    W, nle, max_tokens = 2, 5, 150
+    a, cfg = rank_object(W, nle, H, max_tokens, dt)
+    max_recv = W * max_tokens
+    counts = ragged_counts(rng, nle, max_recv, [max_recv, 0, 65])
+    x = rng.integers(-1, 2, (nle, max_recv, H))
+    w = rng.integers(-1, 2, (nle, H, H))
+    got = run_gemm(a, torch.from_numpy(x).to(dt).to(DEV), counts, torch.from_numpy(w).to(dt).to(DEV))
+    check_padding_untouched(got, counts)
+    name = dtype_name(dt)
+    for le, c in enumerate(counts):
+        want = x[le, :c] @ w[le].T  # |sums| <= H <= 192: integers both 16-bit types hold
+        assert np.array_equal(orc.b16_to_f32(got[le, :c], name), want.astype(np.float32)), f"expert {le}"
+        assert np.array_equal(orc.b16_to_f32(orc.expert_gemm(bits(torch.from_numpy(x[le, :c]).to(dt)),
+                                                             bits(torch.from_numpy(w[le]).to(dt)), name), name),
+                              want.astype(np.float32))
+
+
+def random_case(a, cfg, W, counts, seed, hint=None, check_experts=None):
+    nle, H, dt = cfg.num_experts // W, cfg.hidden_dim, cfg.in_dtype
+    max_recv = W * cfg.max_num_tokens
+    g = torch.Generator(device=DEV).manual_seed(seed)
+    ex = torch.randn(nle, max_recv, H, generator=g, device=DEV, dtype=torch.float32).to(dt)
+    w = (torch.randn(nle, H, H, generator=g, device=DEV, dtype=torch.float32) / H ** 0.5).to(dt)
+    got = run_gemm(a, ex, counts, w, hint)
+    check_padding_untouched(got, counts)
+    name = dtype_name(dt)
+    same = total = 0
+    for le in (range(nle) if check_experts is None else check_experts):
+        c = counts[le]
+        if c == 0:
+            continue
+        xb, wb = bits(ex[le, :c]), bits(w[le])
+        exact, tol = orc.expert_gemm_bound(xb, wb, name)
+        err = np.abs(orc.b16_to_f32(got[le, :c], name).astype(np.float64) - exact)
+        worst = np.unravel_index(np.argmax(err - tol), err.shape)
+        assert (err <= tol).all(), f"expert {le} at {worst}: off by {err[worst]:.3e}, allowed {tol[worst]:.3e}"
+        want32 = orc.expert_gemm(xb, wb, name)
+        assert (np.abs(orc.b16_to_f32(want32, name).astype(np.float64) - exact) <= tol).all()
+        same += int((want32 == got[le, :c]).sum())
+        total += want32.size
+    print(f"  {same}/{total} results equal the float32 oracle to the bit", flush=True)
+    assert same >= 0.98 * total  # they differ where the sum lies next to a rounding boundary
+    return got
+
+
+@pytest.mark.parametrize("name", ["C3", "C4"])
+def test_random_operands_at_workload_sizes(name):
+    print(f"gemm at {name}", flush=True)
+    wl = WORKLOADS[name]
+    W, H, T, K = wl["world_size"], wl["hidden_dim"], wl["max_num_tokens"], wl["experts_per_token"]
+    nle = wl["num_experts"] // W
+    dt = torch.bfloat16
+    a, cfg = rank_object(W, nle, H, T, dt)
+    rng = np.random.default_rng(7)
+    max_recv = W * T
+    # the counts a rank sees at this shape: about W*T*K/num_experts rows per expert, ragged, one empty, one hot
+    counts = [int(c) for c in rng.poisson(W * T * K // wl["num_experts"], nle)]
+    counts[1] = 0
+    counts[2] = min(max_recv, 300)
+    random_case(a, cfg, W, counts, seed=11, hint=sum(counts))
+
+
+@pytest.mark.parametrize("dt", [torch.bfloat16, torch.float16], ids=["bf16", "fp16"])
+def test_hints_and_hot_experts(dt):
+    print(f"gemm hints {dt}", flush=True)
+    W, nle, H, T = 4, 6, 512, 96
+    a, cfg = rank_object(W, nle, H, T, dt)
+    max_recv = W * T
+    counts = [max_recv, 0, 5, max_recv, 131, 64]
+    full = random_case(a, cfg, W, counts, seed=3, hint=sum(counts))
+    for hint in (0, 1, 200, None):  # a hint only sizes the launch: the result does not depend on it
+        assert np.array_equal(run_gemm_same(a, cfg, W, counts, 3, hint), full), f"hint {hint}"
+
+
+def run_gemm_same(a, cfg, W, counts, seed, hint):
+    nle, H, dt = cfg.num_experts // W, cfg.hidden_dim, cfg.in_dtype
+    g = torch.Generator(device=DEV).manual_seed(seed)
+    ex = torch.randn(nle, W * cfg.max_num_tokens, H, generator=g, device=DEV, dtype=torch.float32).to(dt)
+    w = (torch.randn(nle, H, H, generator=g, device=DEV, dtype=torch.float32) / H ** 0.5).to(dt)
+    return run_gemm(a, ex, counts, w, hint)
+
+
+def test_counts_above_the_padding_are_clamped():
+    W, nle, H, T = 2, 2, 128, 8
+    a, cfg = rank_object(W, nle, H, T, torch.bfloat16)
+    got = run_gemm_same(a, cfg, W, [W * T + 50, 3], 5, None)
+    want = run_gemm_same(a, cfg, W, [W * T, 3], 5, None)
+    assert np.array_equal(got, want)
+
+
+def test_both_bindings_give_the_same_bits():
+    W, nle, H, T = 2, 4, 256, 64
+    counts = [128, 7, 0, 90]
+    outs = []
+    for binding in ("ctypes", "ext"):
+        a, cfg = rank_object(W, nle, H, T, torch.bfloat16, binding)
+        outs.append(run_gemm_same(a, cfg, W, counts, 9, None))
+    assert np.array_equal(outs[0], outs[1])
+
+
+def test_unsupported_shapes_raise():
+    a, cfg = rank_object(1, 1, 96, 4, torch.bfloat16)
+    ex = torch.zeros(1, 4, 96, dtype=torch.bfloat16, device=DEV)
+    w = torch.zeros(1, 96, 96, dtype=torch.bfloat16, device=DEV)
+    with pytest.raises(Exception, match="invalid|argument"):
+        a.expert_gemm(ex, torch.tensor([4], dtype=torch.int32, device=DEV), w)
+    with pytest.raises(ValueError, match="weights must be"):
+        a.expert_gemm(ex, torch.tensor([4], dtype=torch.int32, device=DEV), w[:, :64])
