@@ -1555,22 +1555,29 @@ __global__ __launch_bounds__(64 * ROWS) void expert_scale_wave_kernel(
 // expert_y[le, j, :] = expert_x[le, j, :] @ W[le]^T for the valid rows j < expert_num_tokens[le] of
 // the padded expert-major buffers: what stands where all2all/reference.py:262 has the simulated
 // expert. W[le] is [H_out = H, H_in = H] with the input index contiguous (the layout of a linear
-// layer's weight), so that both MFMA operands are read straight from memory in the layout
-// v_mfma_f32_32x32x16 wants: a lane holds 8 consecutive input elements of one row.
+// layer's weight), so the weight operand of v_mfma_f32_32x32x16 is read from memory as it lies: a
+// lane holds consecutive input elements of one output column.
 //
-// With a few dozen rows per expert the problem is bound by streaming the weights (at C4: 3.3 GB of
-// them for 0.2 PFLOP), so the kernel is built to keep weight bytes in flight, not to keep the MFMA
-// pipe full. A workgroup of 4 waves owns a tile of 128 tokens x 128 output columns of one expert,
-// a wave 64 x 64 of it (2 x 2 MFMA tiles, fp32 accumulators in registers), and walks the input
-// dimension 64 elements at a time with the next step's operands requested before the current
-// step's 16 MFMAs are issued. Operands go from global memory to registers: a weight element is used
-// by one workgroup only (an expert with at most 128 rows has one tile of tokens), and the token rows
-// of a tile are re-read by the workgroups of the other column tiles from the L2. No LDS, no barrier
-// in the main loop. The MFMA computes the tile transposed (weights as the A operand, tokens as B),
-// which leaves a lane holding four consecutive output columns of one token: 8-byte stores.
+// With a few dozen rows per expert the problem is bound by streaming the weights (C4: 3.3 GB of
+// them for 0.2 PFLOP), so the kernel is built to keep weight bytes in flight. A workgroup of 4 waves
+// owns 128 output columns x one block of TJ*32 tokens of one expert; a wave owns 32 of the columns
+// for all tokens of the block (TJ MFMA tiles, fp32 accumulators in registers) and walks the input
+// dimension 64 elements at a time. Weights go from global memory straight to registers, each byte
+// to exactly one wave. The token rows are what the 4 waves share: each step's 64 inputs of every
+// token are loaded once per workgroup, parked in LDS, and read from there as the other operand.
+// Both kinds of loads are issued two steps ahead of their use (the vector memory counter retires
+// in order, so the token loads are issued one step earlier than they are parked: waiting for them
+// then never waits for the weights of the next step). One LDS barrier per step.
 //
-// Tiles are numbered over (expert, 128-row block) by a prefix over the device-side counts, so a hot
-// expert is spread over as many workgroups as it has blocks of rows and an empty one costs nothing.
+// The MFMA computes the tile transposed (weights as the A operand, tokens as B), which leaves a lane
+// holding four consecutive output columns of one token: 8-byte stores. Which 8 inputs of a 16-block a
+// lane contributes is the same permutation for both operands (a lane reads 64 contiguous bytes of
+// its weight row per step), so the sums run over the same products as the textbook order.
+//
+// Tiles are numbered over (expert, block of tokens) by a prefix over the device-side counts, so a
+// hot expert is spread over as many workgroups as it has blocks and an empty one costs nothing.
+// Every block of an expert re-reads the expert's weights: TJ = 4 (128 tokens) is used when the
+// caller's row count says blocks of 64 would not hold most experts.
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
@@ -1588,90 +1595,114 @@ template <> struct Mfma32x32x16<MOE_A2A_F16> {
   }
 };
 
-constexpr int GEMM_TILE = 128;   // tokens and output columns per workgroup
-constexpr int GEMM_WAVE = 64;    // tokens and output columns per wave
-constexpr int GEMM_KSTEP = 64;   // input elements per step: a lane reads 64 contiguous bytes of a row
+constexpr int GEMM_COLS = 128;   // output columns per workgroup, 32 per wave
+constexpr int GEMM_KSTEP = 64;   // input elements per step: 8 vectors of 16 bytes per row
 
-template <int DT>
-__global__ __launch_bounds__(BLOCK, 2) void expert_gemm_kernel(
+template <int DT, int TJ>
+__global__ __launch_bounds__(BLOCK, TJ <= 2 ? 4 : 2) void expert_gemm_kernel(
     const b128* __restrict__ expert_x, const int* __restrict__ expert_num_tokens,
     const b128* __restrict__ weights, uint16_t* __restrict__ expert_y, int nle, int max_recv, int H,
     int col_tiles) {
+  constexpr int TOK = TJ * 32;               // tokens per block
+  __shared__ b128 xs[2][TOK * 8];            // two steps of TOK tokens x 8 vectors, vectors swizzled per token
   __shared__ int red[NWAVES];
-  __shared__ int pre[MAX_LOCAL_EXPERTS + 1];  // row blocks before each expert
+  __shared__ int pre[MAX_LOCAL_EXPERTS + 1];  // blocks of tokens before each expert
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
-  expert_prefix_of<NWAVES>(nle, pre, red, [=](int le) {  // blocks of 128 rows per expert
-    return (min(max(expert_num_tokens[le], 0), max_recv) + GEMM_TILE - 1) / GEMM_TILE;
+  const int row_blocks = expert_prefix_of<NWAVES>(nle, pre, red, [=](int le) {
+    return (min(max(expert_num_tokens[le], 0), max_recv) + TOK - 1) / TOK;
   });
-  const int row_blocks = pre[nle];
   const int top = top_step(nle);
-  const int row_vecs = H / 8;                 // 16-byte vectors per row
-  const int wm = wave & 1, wn = wave >> 1;    // this wave's quarter of the tile
-  const int r = lane & 31, kb = lane >> 5;    // MFMA operand layout: row r, input elements kb*8 .. kb*8+7 of a 16-block
+  const int row_vecs = H / 8, steps = H / GEMM_KSTEP;
+  const int r = lane & 31, kb = lane >> 5;  // MFMA operand layout: row r, half kb of the inputs of a step
+
+  // Token vectors this lane loads for the workgroup: slot p = tid + 256*i of a step's TOK*8 slots,
+  // i.e. token p/8, physical vector p%8. A token's vectors are XORed with bits 1..3 of its number so
+  // that the 16 lanes of one LDS access phase (16 tokens, same logical vector) cover all 64 banks.
+  const int load_token = tid >> 3, swz = (load_token >> 1) & 7;
+  const int load_vec = (tid & 7) ^ swz;
+  // Operand reads: token j*32 + r, logical vector kb*4 + q
+  const int read_swz = (r >> 1) & 7;
 
   const int tiles = row_blocks * col_tiles, stride = gridDim.x;
   for (int tile = blockIdx.x; tile < tiles; tile += stride) {
     const int rb = tile / col_tiles, ct = tile - rb * col_tiles;
     const int le = expert_of(pre, nle, top, rb);
     const int rows = min(max(expert_num_tokens[le], 0), max_recv);
-    const int m0 = (rb - pre[le]) * GEMM_TILE + wm * GEMM_WAVE;  // first token of this wave
-    const int n0 = ct * GEMM_TILE + wn * GEMM_WAVE;              // first output column of this wave
-    if (m0 >= rows || n0 >= H) continue;  // (no barrier below: a wave may skip its quarter)
+    const int t0 = (rb - pre[le]) * TOK;                 // first token of the block (t0 < rows)
+    const int n0 = ct * GEMM_COLS + wave * 32;           // first output column of this wave
+    const bool cols_valid = n0 < H;                      // the last tile of columns may be half empty
 
-    // rows of the two operands this lane reads: output columns n0 + i*32 + r of W, tokens m0 + j*32 + r of x
-    const b128* wrow[2];
-    const b128* xrow[2];
+    const b128* wrow = weights + ((size_t)le * H + min(n0 + r, H - 1)) * row_vecs + kb * 4;
+    const b128* xsrc[TJ];
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
-      wrow[i] = weights + ((size_t)le * H + n0 + i * 32 + r) * row_vecs + kb * 4;
-      xrow[i] = expert_x + ((size_t)le * max_recv + min(m0 + i * 32 + r, rows - 1)) * row_vecs + kb * 4;
-    }
-    f32x16 acc[2][2] = {};
-    b128 wv[2][4], xv[2][4];
-    auto fetch = [&](b128 (&wreg)[2][4], b128 (&xreg)[2][4], int k8) {  // k8: step offset in vectors
+    for (int i = 0; i < TJ; ++i)
+      xsrc[i] = expert_x + ((size_t)le * max_recv + min(t0 + load_token + 32 * i, rows - 1)) * row_vecs + load_vec;
+
+    f32x16 acc[TJ] = {};
+    b128 wv[2][4], xv[2][TJ];
+    auto load_w = [&](int set, int step) {
+      const int k8 = min(step, steps - 1) * 8;  // past the end: the last step again, unused
 #pragma unroll
-      for (int i = 0; i < 2; ++i)
-#pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          wreg[i][q] = wrow[i][k8 + q];
-          xreg[i][q] = xrow[i][k8 + q];
-        }
+      for (int q = 0; q < 4; ++q) wv[set][q] = wrow[k8 + q];
     };
-    fetch(wv, xv, 0);
-    for (int k8 = 0; k8 < row_vecs; k8 += GEMM_KSTEP / 8) {
-      b128 wn_[2][4], xn_[2][4];
-      const int next = min(k8 + GEMM_KSTEP / 8, row_vecs - GEMM_KSTEP / 8);  // the last step re-reads itself
-      fetch(wn_, xn_, next);
+    auto load_x = [&](int set, int step) {
+      const int k8 = min(step, steps - 1) * 8;
+#pragma unroll
+      for (int i = 0; i < TJ; ++i) xv[set][i] = xsrc[i][k8];
+    };
+    auto park_x = [&](int set) {  // step s lives in register set s&1 and LDS buffer s&1
+#pragma unroll
+      for (int i = 0; i < TJ; ++i) xs[set][tid + BLOCK * i] = xv[set][i];
+    };
+    auto compute = [&](int set) {
 #pragma unroll
       for (int q = 0; q < 4; ++q)
 #pragma unroll
-        for (int i = 0; i < 2; ++i)
-#pragma unroll
-          for (int j = 0; j < 2; ++j) acc[i][j] = Mfma32x32x16<DT>::mma(wv[i][q], xv[j][q], acc[i][j]);
-#pragma unroll
-      for (int i = 0; i < 2; ++i)
-#pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          wv[i][q] = wn_[i][q];
-          xv[i][q] = xn_[i][q];
+        for (int j = 0; j < TJ; ++j) {
+          const b128 tok = xs[set][(j * 32 + r) * 8 + ((kb * 4 + q) ^ read_swz)];
+          acc[j] = Mfma32x32x16<DT>::mma(wv[set][q], tok, acc[j]);
         }
+    };
+
+    load_x(0, 0);
+    load_w(0, 0);
+    load_x(1, 1);
+    load_w(1, 1);
+    park_x(0);
+    load_x(0, 2);
+    lds_barrier();
+    auto step = [&](int u, int at) {  // step `at` of parity u: register set u, LDS buffer u
+      compute(u);
+      load_w(u, at + 2);
+      park_x(u ^ 1);                  // step at + 1, loaded one step before the weights now in flight
+      load_x(u ^ 1, at + 3);
+      lds_barrier();
+    };
+    // pairs of steps, so that both register sets have fixed names in the loop body; an odd last step
+    // is peeled (inside the loop it would be a path on which an even step follows an even step, and
+    // the compiler would have to wait for the weights as if that happened)
+    int at = 0;
+    for (; at + 1 < steps; at += 2) {
+      step(0, at);
+      step(1, at + 1);
     }
-    // D[n][m] of a 32x32 tile: this lane holds token m = r and output columns (g*8 + kb*4 + 0..3), g < 4
+    if (at < steps) step(0, at);
+
+    // D[n][token] of a 32x32 tile: this lane holds token r and output columns g*8 + kb*4 + 0..3, g < 4
+    if (cols_valid) {
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
-      const int token = m0 + j * 32 + r;
-      if (token < rows) {
-        uint16_t* out = expert_y + ((size_t)le * max_recv + token) * H + n0 + kb * 4;
-#pragma unroll
-        for (int i = 0; i < 2; ++i)
+      for (int j = 0; j < TJ; ++j) {
+        const int token = t0 + j * 32 + r;
+        if (token < rows) {
+          uint16_t* out = expert_y + ((size_t)le * max_recv + token) * H + n0 + kb * 4;
 #pragma unroll
           for (int g = 0; g < 4; ++g) {
-            const f32x16& a = acc[i][j];
-            uint32_t two[2] = {Pair16<DT>::round(a[g * 4 + 0], a[g * 4 + 1]), Pair16<DT>::round(a[g * 4 + 2], a[g * 4 + 3])};
-            two[0] = Pair16<DT>::canonical(two[0]);
-            two[1] = Pair16<DT>::canonical(two[1]);
-            __builtin_memcpy(out + i * 32 + g * 8, two, 8);
+            const f32x16& a = acc[j];
+            uint32_t two[2] = {Pair16<DT>::canonical(Pair16<DT>::round(a[g * 4 + 0], a[g * 4 + 1])),
+                               Pair16<DT>::canonical(Pair16<DT>::round(a[g * 4 + 2], a[g * 4 + 3]))};
+            __builtin_memcpy(out + g * 8, two, 8);
           }
+        }
       }
     }
   }
@@ -2159,29 +2190,39 @@ int moe_a2a_expert_scale(const moe_a2a_shape* s, const void* expert_x,
   return launch_status();
 }
 
+#ifndef MOE_A2A_GEMM_ROWS_FOR_128
+#define MOE_A2A_GEMM_ROWS_FOR_128 40  // rows per expert (mean, from the hint) above which blocks hold 128 tokens
+#endif
+
 int moe_a2a_expert_gemm(const moe_a2a_shape* s, const void* expert_x,
                         const int32_t* expert_num_tokens, int32_t rows_hint, const void* weights,
                         int32_t dtype, void* expert_y, void* stream) {
   if (!shape_ok(s) || rows_hint < 0 || !expert_x || !expert_num_tokens || !weights || !expert_y)
     return MOE_A2A_EINVAL;
   if (dtype != MOE_A2A_F16 && dtype != MOE_A2A_BF16) return MOE_A2A_EINVAL;
-  if (s->hidden_dim % GEMM_KSTEP != 0) return MOE_A2A_EINVAL;  // whole steps of the input, whole wave tiles of columns
+  if (s->hidden_dim % GEMM_KSTEP != 0) return MOE_A2A_EINVAL;  // whole steps of the input
   if (!all_aligned(16, expert_x, weights, expert_y)) return MOE_A2A_EALIGN;
   const int nle = s->num_experts / s->world_size;
   if (nle > MAX_LOCAL_EXPERTS) return MOE_A2A_EINVAL;
   const long long max_recv = (long long)s->max_num_tokens * s->world_size;
-  const int col_tiles = (s->hidden_dim + GEMM_TILE - 1) / GEMM_TILE;
-  // every expert can end in a partly filled block of rows; the kernel strides over what the hint misses
-  const long long row_blocks = (long long)rows_hint / GEMM_TILE + nle;
-  if ((max_recv / GEMM_TILE + 1) * nle * col_tiles > INT_MAX / 2) return MOE_A2A_EINVAL;
+  const int col_tiles = (s->hidden_dim + GEMM_COLS - 1) / GEMM_COLS;
+  const int tj = (long long)rows_hint > (long long)MOE_A2A_GEMM_ROWS_FOR_128 * nle ? 4 : 2;
+  // every expert can end in a partly filled block of tokens; the kernel strides over what the hint misses
+  const long long row_blocks = (long long)rows_hint / (tj * 32) + nle;
+  if ((max_recv / 64 + 1) * nle * col_tiles > INT_MAX / 2) return MOE_A2A_EINVAL;
   const int grid = mover_blocks(row_blocks * col_tiles);
   hipStream_t st = (hipStream_t)stream;
-#define LAUNCH_G(DT)                                                                         \
-  expert_gemm_kernel<DT><<<grid, BLOCK, 0, st>>>((const b128*)expert_x, expert_num_tokens,   \
-                                                 (const b128*)weights, (uint16_t*)expert_y,  \
-                                                 nle, (int)max_recv, s->hidden_dim, col_tiles)
-  if (dtype == MOE_A2A_BF16) LAUNCH_G(MOE_A2A_BF16);
-  else LAUNCH_G(MOE_A2A_F16);
+#define LAUNCH_G(DT, TJ)                                                                         \
+  expert_gemm_kernel<DT, TJ><<<grid, BLOCK, 0, st>>>((const b128*)expert_x, expert_num_tokens,   \
+                                                     (const b128*)weights, (uint16_t*)expert_y,  \
+                                                     nle, (int)max_recv, s->hidden_dim, col_tiles)
+  if (dtype == MOE_A2A_BF16) {
+    if (tj == 2) LAUNCH_G(MOE_A2A_BF16, 2);
+    else LAUNCH_G(MOE_A2A_BF16, 4);
+  } else {
+    if (tj == 2) LAUNCH_G(MOE_A2A_F16, 2);
+    else LAUNCH_G(MOE_A2A_F16, 4);
+  }
 #undef LAUNCH_G
   return launch_status();
 }
