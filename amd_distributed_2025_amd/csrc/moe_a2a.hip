@@ -1555,24 +1555,33 @@ __global__ __launch_bounds__(64 * ROWS) void expert_scale_wave_kernel(
 // expert_y[le, j, :] = expert_x[le, j, :] @ W[le]^T for the valid rows j < expert_num_tokens[le] of
 // the padded expert-major buffers: what stands where all2all/reference.py:262 has the simulated
 // expert. W[le] is [H_out = H, H_in = H] with the input index contiguous (the layout of a linear
-// layer's weight), so the weight operand of v_mfma_f32_32x32x16 is read from memory as it lies: a
-// lane holds consecutive input elements of one output column.
+// layer's weight).
 //
 // With a few dozen rows per expert the problem is bound by streaming the weights (C4: 3.3 GB of
-// them for 0.2 PFLOP), so the kernel is built to keep weight bytes in flight. A workgroup of 4 waves
-// owns 128 output columns x one block of TJ*32 tokens of one expert; a wave owns 32 of the columns
-// for all tokens of the block (TJ MFMA tiles, fp32 accumulators in registers) and walks the input
-// dimension 64 elements at a time. Weights go from global memory straight to registers, each byte
-// to exactly one wave. The token rows are what the 4 waves share: each step's 64 inputs of every
-// token are loaded once per workgroup, parked in LDS, and read from there as the other operand.
-// Both kinds of loads are issued two steps ahead of their use (the vector memory counter retires
-// in order, so the token loads are issued one step earlier than they are parked: waiting for them
-// then never waits for the weights of the next step). One LDS barrier per step.
+// them for 0.2 PFLOP), so the kernel is built to keep weight bytes in flight and to ask for them in
+// whole cache lines. A workgroup of 4 waves owns 128 output columns x one block of TJ*32 tokens of
+// one expert; a wave owns 32 of the columns for all tokens of the block (TJ tiles of
+// v_mfma_f32_32x32x16, fp32 accumulators in registers) and walks the input dimension 64 elements
+// (128 bytes of every row) at a time.
+//
+// Weights: the MFMA wants a lane to hold inputs of ONE output column, which read from memory as
+// it lies makes every load instruction touch 32 different lines, a quarter of each (measured: 4.0
+// TB/s against 5.6 with the same bytes requested line by line). So a wave loads its 32 x 128 bytes
+// of a step with 8 lanes per line, drops them into 4 KB of LDS of its own, and picks the operands
+// up from there in MFMA layout. No barrier is involved: a wave's LDS operations execute in order.
+// Tokens: the rows of the block are what the 4 waves share. Each step's 128 bytes of every token
+// are loaded once per workgroup, parked in LDS and read from there by all four: one LDS barrier per
+// step. Both kinds of loads are issued DEPTH steps ahead of their use; the vector memory counter
+// retires in order, so the token loads run one step ahead of the weights: waiting for the tokens
+// that are parked next never waits for the weights issued after them.
+// LDS layout of both: row-major 128-byte rows, the eight 16-byte vectors of a row XORed with bits
+// 1..3 of the row number, which makes the parking writes (8 lanes per row) and the operand reads
+// (16 rows, same vector) hit all 64 banks once per 16 lanes.
 //
 // The MFMA computes the tile transposed (weights as the A operand, tokens as B), which leaves a lane
 // holding four consecutive output columns of one token: 8-byte stores. Which 8 inputs of a 16-block a
-// lane contributes is the same permutation for both operands (a lane reads 64 contiguous bytes of
-// its weight row per step), so the sums run over the same products as the textbook order.
+// lane contributes is the same permutation for both operands, so the sums run over the same
+// products as the textbook order.
 //
 // Tiles are numbered over (expert, block of tokens) by a prefix over the device-side counts, so a
 // hot expert is spread over as many workgroups as it has blocks and an empty one costs nothing.
@@ -1595,98 +1604,152 @@ template <> struct Mfma32x32x16<MOE_A2A_F16> {
   }
 };
 
+#ifndef MOE_A2A_GEMM_OCC
+#define MOE_A2A_GEMM_OCC 4
+#endif
+#ifndef MOE_A2A_GEMM_DEPTH
+#define MOE_A2A_GEMM_DEPTH 2
+#endif
 constexpr int GEMM_COLS = 128;   // output columns per workgroup, 32 per wave
 constexpr int GEMM_KSTEP = 64;   // input elements per step: 8 vectors of 16 bytes per row
+constexpr int GEMM_DEPTH = MOE_A2A_GEMM_DEPTH;  // steps between a load and its use
 
 template <int DT, int TJ>
-__global__ __launch_bounds__(BLOCK, TJ <= 2 ? 4 : 2) void expert_gemm_kernel(
+__global__ __launch_bounds__(BLOCK, TJ <= 2 ? MOE_A2A_GEMM_OCC : 2) void expert_gemm_kernel(
     const b128* __restrict__ expert_x, const int* __restrict__ expert_num_tokens,
     const b128* __restrict__ weights, uint16_t* __restrict__ expert_y, int nle, int max_recv, int H,
     int col_tiles) {
   constexpr int TOK = TJ * 32;               // tokens per block
-  __shared__ b128 xs[2][TOK * 8];            // two steps of TOK tokens x 8 vectors, vectors swizzled per token
+  constexpr int D = GEMM_DEPTH;
+  __shared__ b128 xs[D][TOK * 8];            // D steps of TOK tokens x 8 vectors
+  __shared__ b128 ws[NWAVES][32 * 8];        // per wave: one step of its 32 weight rows x 8 vectors
   __shared__ int red[NWAVES];
-  __shared__ int pre[MAX_LOCAL_EXPERTS + 1];  // blocks of tokens before each expert
+  __shared__ int home[2];
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
-  const int row_blocks = expert_prefix_of<NWAVES>(nle, pre, red, [=](int le) {
-    return (min(max(expert_num_tokens[le], 0), max_recv) + TOK - 1) / TOK;
-  });
-  const int top = top_step(nle);
   const int row_vecs = H / 8, steps = H / GEMM_KSTEP;
-  const int r = lane & 31, kb = lane >> 5;  // MFMA operand layout: row r, half kb of the inputs of a step
 
-  // Token vectors this lane loads for the workgroup: slot p = tid + 256*i of a step's TOK*8 slots,
-  // i.e. token p/8, physical vector p%8. A token's vectors are XORed with bits 1..3 of its number so
-  // that the 16 lanes of one LDS access phase (16 tokens, same logical vector) cover all 64 banks.
-  const int load_token = tid >> 3, swz = (load_token >> 1) & 7;
-  const int load_vec = (tid & 7) ^ swz;
-  // Operand reads: token j*32 + r, logical vector kb*4 + q
-  const int read_swz = (r >> 1) & 7;
+  // Blocks of tokens per expert, summed over the run of experts this thread owns and scanned over
+  // the workgroup: block number g of the launch belongs to the thread with begin <= g < begin + mine.
+  auto blocks_of = [=](int le) { return (min(max(expert_num_tokens[le], 0), max_recv) + TOK - 1) / TOK; };
+  const int per = (nle + BLOCK - 1) / BLOCK;
+  const int run_b = min(tid * per, nle), run_e = min(run_b + per, nle);
+  int mine = 0;
+  for (int le = run_b; le < run_e; ++le) mine += blocks_of(le);
+  int begin, row_blocks;
+  {
+    const int inc = wave_inclusive_scan(mine);
+    if (lane == 63) red[wave] = inc;
+    lds_barrier();
+    int off = 0, total = 0;
+#pragma unroll
+    for (int w = 0; w < NWAVES; ++w) {
+      off += w < wave ? red[w] : 0;
+      total += red[w];
+    }
+    begin = off + inc - mine;
+    row_blocks = total;
+  }
+
+  // Loads are 8 lanes per 128-byte row: lane l of a wave takes row l/8 (+ 8 per further load) and
+  // the vector of that row that belongs in physical slot l%8.
+  const int sub = lane >> 3, slot = lane & 7;
+  // operand reads: row r of the tile, half kb of the step's inputs, logical vector kb*4 + q
+  const int r = lane & 31, kb = lane >> 5, read_swz = (r >> 1) & 7;
 
   const int tiles = row_blocks * col_tiles, stride = gridDim.x;
   for (int tile = blockIdx.x; tile < tiles; tile += stride) {
     const int rb = tile / col_tiles, ct = tile - rb * col_tiles;
-    const int le = expert_of(pre, nle, top, rb);
-    const int rows = min(max(expert_num_tokens[le], 0), max_recv);
-    const int t0 = (rb - pre[le]) * TOK;                 // first token of the block (t0 < rows)
-    const int n0 = ct * GEMM_COLS + wave * 32;           // first output column of this wave
+    if (begin <= rb && rb < begin + mine) {  // one thread: walk its run to the expert of block rb
+      int le = run_b, first = begin;
+      for (;; ++le) {
+        const int n = blocks_of(le);
+        if (rb < first + n) break;
+        first += n;
+      }
+      home[0] = le;
+      home[1] = first;
+    }
+    lds_barrier();  // (the next write to `home` comes after the barriers of the steps below)
+    // (uniform values are pinned to scalar registers: the bases below then cost no vector registers)
+    const int le = __builtin_amdgcn_readfirstlane(home[0]);
+    const int rows = min(max(__builtin_amdgcn_readfirstlane(expert_num_tokens[le]), 0), max_recv);
+    const int t0 = (rb - __builtin_amdgcn_readfirstlane(home[1])) * TOK;  // first token of the block (t0 < rows)
+    const int n0 = ct * GEMM_COLS + __builtin_amdgcn_readfirstlane(wave) * 32;  // first output column of this wave
     const bool cols_valid = n0 < H;                      // the last tile of columns may be half empty
+    const int nw = min(n0, H - 32);                      // (a wave without columns reads valid memory)
 
-    const b128* wrow = weights + ((size_t)le * H + min(n0 + r, H - 1)) * row_vecs + kb * 4;
-    const b128* xsrc[TJ];
+    // weights: load i takes rows sub + 8*i of the wave's 32; tokens: load i takes tokens tid/8 + 32*i.
+    // Offsets are in vectors from a base that is uniform over the wave and moves with the step.
+    const b128* wbase = weights + ((size_t)le * H + nw) * row_vecs;
+    const b128* xbase = expert_x + ((size_t)le * max_recv + t0) * row_vecs;
+    int woff[4], wslot[4], xoff[TJ];
 #pragma unroll
-    for (int i = 0; i < TJ; ++i)
-      xsrc[i] = expert_x + ((size_t)le * max_recv + min(t0 + load_token + 32 * i, rows - 1)) * row_vecs + load_vec;
+    for (int i = 0; i < 4; ++i) {
+      const int row = sub + 8 * i;
+      woff[i] = row * row_vecs + (slot ^ ((row >> 1) & 7));
+      wslot[i] = row * 8 + slot;
+    }
+    const int xrow = tid >> 3, xvec = slot ^ ((xrow >> 1) & 7);  // (32*i does not change bits 1..3)
+#pragma unroll
+    for (int i = 0; i < TJ; ++i) xoff[i] = min(xrow + 32 * i, rows - 1 - t0) * row_vecs + xvec;
 
     f32x16 acc[TJ] = {};
-    b128 wv[2][4], xv[2][TJ];
+    b128 wv[D][4], xv[D][TJ];
     auto load_w = [&](int set, int step) {
-      const int k8 = min(step, steps - 1) * 8;  // past the end: the last step again, unused
+      const b128* at = wbase + min(step, steps - 1) * 8;  // past the end: the last step again, unused
 #pragma unroll
-      for (int q = 0; q < 4; ++q) wv[set][q] = wrow[k8 + q];
+      for (int i = 0; i < 4; ++i) wv[set][i] = at[woff[i]];
     };
     auto load_x = [&](int set, int step) {
-      const int k8 = min(step, steps - 1) * 8;
+      const b128* at = xbase + min(step, steps - 1) * 8;
 #pragma unroll
-      for (int i = 0; i < TJ; ++i) xv[set][i] = xsrc[i][k8];
+      for (int i = 0; i < TJ; ++i) xv[set][i] = at[xoff[i]];
     };
-    auto park_x = [&](int set) {  // step s lives in register set s&1 and LDS buffer s&1
+    auto park_x = [&](int set) {
 #pragma unroll
       for (int i = 0; i < TJ; ++i) xs[set][tid + BLOCK * i] = xv[set][i];
     };
     auto compute = [&](int set) {
 #pragma unroll
+      for (int i = 0; i < 4; ++i) ws[wave][wslot[i]] = wv[set][i];
+      b128 a[4];
+#pragma unroll
+      for (int q = 0; q < 4; ++q) a[q] = ws[wave][r * 8 + ((kb * 4 + q) ^ read_swz)];
+#pragma unroll
       for (int q = 0; q < 4; ++q)
 #pragma unroll
         for (int j = 0; j < TJ; ++j) {
           const b128 tok = xs[set][(j * 32 + r) * 8 + ((kb * 4 + q) ^ read_swz)];
-          acc[j] = Mfma32x32x16<DT>::mma(wv[set][q], tok, acc[j]);
+          acc[j] = Mfma32x32x16<DT>::mma(a[q], tok, acc[j]);
         }
     };
-
-    load_x(0, 0);
-    load_w(0, 0);
-    load_x(1, 1);
-    load_w(1, 1);
-    park_x(0);
-    load_x(0, 2);
-    lds_barrier();
-    auto step = [&](int u, int at) {  // step `at` of parity u: register set u, LDS buffer u
+    auto step = [&](int u, int at) {  // step `at`, which lives in register set and LDS buffer u = at % D
       compute(u);
-      load_w(u, at + 2);
-      park_x(u ^ 1);                  // step at + 1, loaded one step before the weights now in flight
-      load_x(u ^ 1, at + 3);
+      load_w(u, at + D);
+      park_x((u + 1) % D);            // step at + 1, loaded one step before the weights now in flight
+      load_x((u + 1) % D, at + 1 + D);
       lds_barrier();
     };
-    // pairs of steps, so that both register sets have fixed names in the loop body; an odd last step
-    // is peeled (inside the loop it would be a path on which an even step follows an even step, and
+
+#pragma unroll
+    for (int i = 0; i < D; ++i) {
+      load_x(i, i);
+      load_w(i, i);
+    }
+    park_x(0);
+    load_x(0, D);
+    lds_barrier();
+    // D steps per trip, so that the register sets have fixed names in the loop body; the last
+    // steps % D are peeled (inside the loop they would be paths on which set 0 follows set 0, and
     // the compiler would have to wait for the weights as if that happened)
     int at = 0;
-    for (; at + 1 < steps; at += 2) {
-      step(0, at);
-      step(1, at + 1);
+    for (; at + D <= steps; at += D) {
+#pragma unroll
+      for (int u = 0; u < D; ++u) step(u, at + u);
     }
-    if (at < steps) step(0, at);
+#pragma unroll
+    for (int u = 0; u < D - 1; ++u)
+      if (at + u < steps) step(u, at + u);
 
     // D[n][token] of a 32x32 tile: this lane holds token r and output columns g*8 + kb*4 + 0..3, g < 4
     if (cols_valid) {
@@ -1697,9 +1760,9 @@ __global__ __launch_bounds__(BLOCK, TJ <= 2 ? 4 : 2) void expert_gemm_kernel(
           uint16_t* out = expert_y + ((size_t)le * max_recv + token) * H + n0 + kb * 4;
 #pragma unroll
           for (int g = 0; g < 4; ++g) {
-            const f32x16& a = acc[j];
-            uint32_t two[2] = {Pair16<DT>::canonical(Pair16<DT>::round(a[g * 4 + 0], a[g * 4 + 1])),
-                               Pair16<DT>::canonical(Pair16<DT>::round(a[g * 4 + 2], a[g * 4 + 3]))};
+            const f32x16& c = acc[j];
+            uint32_t two[2] = {Pair16<DT>::canonical(Pair16<DT>::round(c[g * 4 + 0], c[g * 4 + 1])),
+                               Pair16<DT>::canonical(Pair16<DT>::round(c[g * 4 + 2], c[g * 4 + 3]))};
             __builtin_memcpy(out + g * 8, two, 8);
           }
         }
@@ -2203,7 +2266,6 @@ int moe_a2a_expert_gemm(const moe_a2a_shape* s, const void* expert_x,
   if (s->hidden_dim % GEMM_KSTEP != 0) return MOE_A2A_EINVAL;  // whole steps of the input
   if (!all_aligned(16, expert_x, weights, expert_y)) return MOE_A2A_EALIGN;
   const int nle = s->num_experts / s->world_size;
-  if (nle > MAX_LOCAL_EXPERTS) return MOE_A2A_EINVAL;
   const long long max_recv = (long long)s->max_num_tokens * s->world_size;
   const int col_tiles = (s->hidden_dim + GEMM_COLS - 1) / GEMM_COLS;
   const int tj = (long long)rows_hint > (long long)MOE_A2A_GEMM_ROWS_FOR_128 * nle ? 4 : 2;
