@@ -2254,7 +2254,7 @@ int moe_a2a_expert_scale(const moe_a2a_shape* s, const void* expert_x,
 }
 
 #ifndef MOE_A2A_GEMM_ROWS_FOR_128
-#define MOE_A2A_GEMM_ROWS_FOR_128 40  // rows per expert (mean, from the hint) above which blocks hold 128 tokens
+#define MOE_A2A_GEMM_ROWS_FOR_128 48  // rows per expert (mean, from the hint) above which blocks hold 128 tokens
 #endif
 
 int moe_a2a_expert_gemm(const moe_a2a_shape* s, const void* expert_x,

@@ -24,7 +24,10 @@ the step leaves it. The cost of one of them is that time minus the time of the s
 hot-path figure for every rank of the job (their received row counts differ); `cpu_baseline` is the
 row-by-row torch-CPU statement of the same step timed on this box's
 host cores, with the vectorised numpy statement beside it; `custom_kernel_wall_us` is one call of the
-reference's entry point (which steps all ranks of the job on this one GPU).
+reference's entry point (which steps all ranks of the job on this one GPU). `expert_gemm` is the
+grouped GEMM a model would run between the two halves, on this rank's expert-major rows and random
+weights: one launch between HIP events, priced against HBM peak (it streams every weight once) with
+its matrix rate beside it.
 """
 from __future__ import annotations
 
@@ -41,6 +44,7 @@ if str(ROOT) not in sys.path:
     sys.path.insert(0, str(ROOT))
 
 HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published
+MFMA_PEAK_TFLOPS = 2500.0  # MI355X dense bf16/fp16 matrix rate, published
 META_BYTES = 20
 # HBM bytes per launch from rocprofv3 FETCH_SIZE / WRITE_SIZE, with the build they were measured on
 TRAFFIC_FILE = ROOT / "profiles" / "hbm_traffic.json"
@@ -61,6 +65,7 @@ def parse_args():
                     help="repetitions of the launches inside each timing graph")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="target CPU time of the cpu_baseline sample")
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
+    ap.add_argument("--no-gemm", action="store_true", help="skip the grouped GEMM row")
     ap.add_argument("--no-rank-sweep", action="store_true", help="time only --rank, not every rank of the job")
     ap.add_argument("--no-placement-plan", action="store_true",
                     help="combine_send ranks its rows by scanning instead of using dispatch_recv's plan")
@@ -322,6 +327,45 @@ def main():
     set_peer_inputs(None)
     out["custom_kernel_wall_us"] = round(statistics.median(walls[2:]), 1)
     out["custom_kernel_matches_step"] = bool(torch.equal(yk, ys0[r0]))
+
+    # ---- the expert computation a model runs between the two halves: the grouped GEMM over this
+    # rank's expert-major rows (random weights; the stand-in of the reference stays in the step above)
+    if not args.no_gemm and H % 64 == 0 and cfg.in_dtype == cfg.out_dtype:
+        a, g = lw.ranks[r0], lw.trace[r0]
+        nle = a.num_local_experts
+        gen = torch.Generator(device=dev).manual_seed(args.seed)
+        wts = torch.empty(nle, H, H, dtype=cfg.in_dtype, device=dev)
+        for le in range(nle):  # (one expert at a time: the fp32 draw of all of them would not be small)
+            wts[le] = (torch.randn(H, H, generator=gen, device=dev) / H ** 0.5).to(cfg.in_dtype)
+        ex, num = g["expert_x"], g["expert_num_tokens"]
+        counts = num.cpu().tolist()
+        ev = [torch.cuda.Event(enable_timing=True) for _ in range(2)]
+        times = []
+        for i in range(12):
+            ev[0].record()
+            ey = a.expert_gemm(ex, num, wts, R)
+            ev[1].record()
+            ev[1].synchronize()
+            if i >= 2:
+                times.append(ev[0].elapsed_time(ev[1]) * 1e3)
+        gemm_us = statistics.median(times)
+        le = max(range(nle), key=lambda i: counts[i])
+        want = ex[le, : counts[le]].float() @ wts[le].float().T
+        err = (ey[le, : counts[le]].float() - want).abs().max().item()
+        gemm_bytes = nle * H * H * 2 + 2 * R * H * 2   # every weight once, valid rows read and written
+        gemm_flop = 2 * R * H * H
+        out["expert_gemm"] = {
+            "us": round(gemm_us, 1), "rows": R, "rows_per_expert_max": max(counts), "experts": nle,
+            "weights_bytes": nle * H * H * 2, "alg_bytes": gemm_bytes, "flop": gemm_flop,
+            "roofline": {"bound": "hbm", "achieved": round(gemm_bytes / gemm_us * 1e-3, 1), "peak": HBM_PEAK_GBPS,
+                         "unit": "GB/s", "frac": round(gemm_bytes / gemm_us * 1e-3 / HBM_PEAK_GBPS, 4)},
+            "tflops": round(gemm_flop / gemm_us * 1e-6, 1),
+            "frac_of_mfma_peak": round(gemm_flop / gemm_us * 1e-6 / MFMA_PEAK_TFLOPS, 4),
+            "mfma_peak_tflops": MFMA_PEAK_TFLOPS,
+            "max_abs_err_vs_fp32_matmul": err,
+            "measure": "HIP events around single launches, median of 10",
+        }
+        del wts
 
     # ---- CPU baseline: the row-by-row torch statement of the same step on the host cores
     if not args.no_cpu:
