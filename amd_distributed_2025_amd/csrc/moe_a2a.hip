@@ -1610,6 +1610,7 @@ template <> struct Mfma32x32x16<MOE_A2A_F16> {
 #ifndef MOE_A2A_GEMM_DEPTH
 #define MOE_A2A_GEMM_DEPTH 2
 #endif
+constexpr int BUFFER_RAW_32BIT = 0x00020000;  // word 3 of a gfx9 buffer descriptor: raw buffer of 32-bit data
 constexpr int GEMM_COLS = 128;   // output columns per workgroup, 32 per wave
 constexpr int GEMM_KSTEP = 64;   // input elements per step: 8 vectors of 16 bytes per row
 constexpr int GEMM_DEPTH = MOE_A2A_GEMM_DEPTH;  // steps between a load and its use
@@ -1679,31 +1680,38 @@ __global__ __launch_bounds__(BLOCK, TJ <= 2 ? MOE_A2A_GEMM_OCC : 2) void expert_
     const int nw = min(n0, H - 32);                      // (a wave without columns reads valid memory)
 
     // weights: load i takes rows sub + 8*i of the wave's 32; tokens: load i takes tokens tid/8 + 32*i.
-    // Offsets are in vectors from a base that is uniform over the wave and moves with the step.
-    const b128* wbase = weights + ((size_t)le * H + nw) * row_vecs;
-    const b128* xbase = expert_x + ((size_t)le * max_recv + t0) * row_vecs;
+    // Both go through buffer descriptors (base and extent in scalar registers, a 32-bit byte offset
+    // per lane, the step's offset as the scalar operand). The extent of the token buffer ends with
+    // the expert's last valid row: lanes that would load tokens past it get zeros and cause no
+    // traffic. Tiles of 32 tokens with no valid token are skipped altogether.
+    const int live = rows - t0;  // valid tokens of this block, > 0
+    const int row_bytes = H * 2;
+    const __amdgpu_buffer_rsrc_t wbuf = __builtin_amdgcn_make_buffer_rsrc(
+        (void*)(weights + ((size_t)le * H + nw) * row_vecs), 0, 32 * row_bytes, BUFFER_RAW_32BIT);
+    const __amdgpu_buffer_rsrc_t xbuf = __builtin_amdgcn_make_buffer_rsrc(
+        (void*)(expert_x + ((size_t)le * max_recv + t0) * row_vecs), 0, min(live, TOK) * row_bytes, BUFFER_RAW_32BIT);
     int woff[4], wslot[4], xoff[TJ];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const int row = sub + 8 * i;
-      woff[i] = row * row_vecs + (slot ^ ((row >> 1) & 7));
+      woff[i] = row * row_bytes + (slot ^ ((row >> 1) & 7)) * 16;
       wslot[i] = row * 8 + slot;
     }
     const int xrow = tid >> 3, xvec = slot ^ ((xrow >> 1) & 7);  // (32*i does not change bits 1..3)
 #pragma unroll
-    for (int i = 0; i < TJ; ++i) xoff[i] = min(xrow + 32 * i, rows - 1 - t0) * row_vecs + xvec;
+    for (int i = 0; i < TJ; ++i) xoff[i] = (xrow + 32 * i) * row_bytes + xvec * 16;
 
     f32x16 acc[TJ] = {};
     b128 wv[D][4], xv[D][TJ];
     auto load_w = [&](int set, int step) {
-      const b128* at = wbase + min(step, steps - 1) * 8;  // past the end: the last step again, unused
+      const int k = min(step, steps - 1) * (GEMM_KSTEP * 2);  // past the end: the last step again, unused
 #pragma unroll
-      for (int i = 0; i < 4; ++i) wv[set][i] = at[woff[i]];
+      for (int i = 0; i < 4; ++i) wv[set][i] = __builtin_amdgcn_raw_buffer_load_b128(wbuf, woff[i], k, 0);
     };
     auto load_x = [&](int set, int step) {
-      const b128* at = xbase + min(step, steps - 1) * 8;
+      const int k = min(step, steps - 1) * (GEMM_KSTEP * 2);
 #pragma unroll
-      for (int i = 0; i < TJ; ++i) xv[set][i] = at[xoff[i]];
+      for (int i = 0; i < TJ; ++i) xv[set][i] = __builtin_amdgcn_raw_buffer_load_b128(xbuf, xoff[i], k, 0);
     };
     auto park_x = [&](int set) {
 #pragma unroll
@@ -1719,8 +1727,10 @@ __global__ __launch_bounds__(BLOCK, TJ <= 2 ? MOE_A2A_GEMM_OCC : 2) void expert_
       for (int q = 0; q < 4; ++q)
 #pragma unroll
         for (int j = 0; j < TJ; ++j) {
-          const b128 tok = xs[set][(j * 32 + r) * 8 + ((kb * 4 + q) ^ read_swz)];
-          acc[j] = Mfma32x32x16<DT>::mma(a[q], tok, acc[j]);
+          if (j * 32 < live) {
+            const b128 tok = xs[set][(j * 32 + r) * 8 + ((kb * 4 + q) ^ read_swz)];
+            acc[j] = Mfma32x32x16<DT>::mma(a[q], tok, acc[j]);
+          }
         }
     };
     auto step = [&](int u, int at) {  // step `at`, which lives in register set and LDS buffer u = at % D
