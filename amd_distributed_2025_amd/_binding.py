@@ -78,6 +78,11 @@ class CtypesBinding:
         _lib.call("moe_a2a_expert_gemm", C.byref(shape), _ptr(expert_x), _ptr(expert_num_tokens), rows_hint,
                   _ptr(weights), _DT[expert_x.dtype], _ptr(expert_y), C.c_void_p(stream))
 
+    def linear(self, input, weight, bias, output, stream):
+        m, k = input.shape
+        _lib.call("moe_a2a_linear", _ptr(input), _ptr(weight), _ptr(bias), m, weight.shape[0], k, _DT[input.dtype],
+                  _ptr(output), C.c_void_p(stream))
+
     def exchange_local(self, world_size, hidden_dim, send_buf, send_meta, send_counts, dst_rank, recv_buf,
                        recv_meta, recv_counts, src_rank, rows_hint, stream):
         _lib.call("moe_a2a_exchange_local", world_size, hidden_dim, _ptr(send_buf), _ptr(send_meta),
@@ -131,6 +136,9 @@ class ExtBinding:
     def expert_gemm(self, shape, expert_x, expert_num_tokens, rows_hint, weights, expert_y, stream):
         self._m.a2a_expert_gemm(self._shape(shape), expert_x, expert_num_tokens, rows_hint, weights, expert_y,
                                 stream)
+
+    def linear(self, input, weight, bias, output, stream):
+        self._m.a2a_linear(input, weight, bias, output, stream)
 
     def exchange_local(self, world_size, hidden_dim, send_buf, send_meta, send_counts, dst_rank, recv_buf,
                        recv_meta, recv_counts, src_rank, rows_hint, stream):

@@ -1605,7 +1605,7 @@ template <> struct Mfma32x32x16<MOE_A2A_F16> {
 };
 
 #ifndef MOE_A2A_GEMM_OCC
-#define MOE_A2A_GEMM_OCC 4
+#define MOE_A2A_GEMM_OCC 3
 #endif
 #ifndef MOE_A2A_GEMM_DEPTH
 #define MOE_A2A_GEMM_DEPTH 2
@@ -1615,11 +1615,13 @@ constexpr int GEMM_COLS = 128;   // output columns per workgroup, 32 per wave
 constexpr int GEMM_KSTEP = 64;   // input elements per step: 8 vectors of 16 bytes per row
 constexpr int GEMM_DEPTH = MOE_A2A_GEMM_DEPTH;  // steps between a load and its use
 
+// x [groups, max_rows, K], w [groups, N, K], bias [groups, N] or null, y [groups, max_rows, N];
+// rows_of_group null: every group has max_rows rows (a plain dense product when groups == 1).
 template <int DT, int TJ>
 __global__ __launch_bounds__(BLOCK, TJ <= 2 ? MOE_A2A_GEMM_OCC : 2) void expert_gemm_kernel(
     const b128* __restrict__ expert_x, const int* __restrict__ expert_num_tokens,
-    const b128* __restrict__ weights, uint16_t* __restrict__ expert_y, int nle, int max_recv, int H,
-    int col_tiles) {
+    const b128* __restrict__ weights, const uint16_t* __restrict__ bias, uint16_t* __restrict__ expert_y,
+    int nle, int max_recv, int N, int K, int col_tiles) {
   constexpr int TOK = TJ * 32;               // tokens per block
   constexpr int D = GEMM_DEPTH;
   __shared__ b128 xs[D][TOK * 8];            // D steps of TOK tokens x 8 vectors
@@ -1627,11 +1629,13 @@ __global__ __launch_bounds__(BLOCK, TJ <= 2 ? MOE_A2A_GEMM_OCC : 2) void expert_
   __shared__ int red[NWAVES];
   __shared__ int home[2];
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
-  const int row_vecs = H / 8, steps = H / GEMM_KSTEP;
+  const int row_vecs = K / 8, steps = (K + GEMM_KSTEP - 1) / GEMM_KSTEP;
+  const int tail_vecs = row_vecs - (steps - 1) * 8;  // vectors of a row in the last step, 1..8
+  auto rows_of = [=](int le) { return expert_num_tokens ? min(max(expert_num_tokens[le], 0), max_recv) : max_recv; };
 
   // Blocks of tokens per expert, summed over the run of experts this thread owns and scanned over
   // the workgroup: block number g of the launch belongs to the thread with begin <= g < begin + mine.
-  auto blocks_of = [=](int le) { return (min(max(expert_num_tokens[le], 0), max_recv) + TOK - 1) / TOK; };
+  auto blocks_of = [=](int le) { return (rows_of(le) + TOK - 1) / TOK; };
   const int per = (nle + BLOCK - 1) / BLOCK;
   const int run_b = min(tid * per, nle), run_e = min(run_b + per, nle);
   int mine = 0;
@@ -1673,45 +1677,56 @@ __global__ __launch_bounds__(BLOCK, TJ <= 2 ? MOE_A2A_GEMM_OCC : 2) void expert_
     lds_barrier();  // (the next write to `home` comes after the barriers of the steps below)
     // (uniform values are pinned to scalar registers: the bases below then cost no vector registers)
     const int le = __builtin_amdgcn_readfirstlane(home[0]);
-    const int rows = min(max(__builtin_amdgcn_readfirstlane(expert_num_tokens[le]), 0), max_recv);
+    const int rows = __builtin_amdgcn_readfirstlane(rows_of(le));
     const int t0 = (rb - __builtin_amdgcn_readfirstlane(home[1])) * TOK;  // first token of the block (t0 < rows)
     const int n0 = ct * GEMM_COLS + __builtin_amdgcn_readfirstlane(wave) * 32;  // first output column of this wave
-    const bool cols_valid = n0 < H;                      // the last tile of columns may be half empty
-    const int nw = min(n0, H - 32);                      // (a wave without columns reads valid memory)
+    const bool cols_valid = n0 < N;                      // the last tile of columns may be partly empty
+    const int nw = min(n0, N - 32);                      // (a wave without columns reads valid memory)
 
     // weights: load i takes rows sub + 8*i of the wave's 32; tokens: load i takes tokens tid/8 + 32*i.
     // Both go through buffer descriptors (base and extent in scalar registers, a 32-bit byte offset
     // per lane, the step's offset as the scalar operand). The extent of the token buffer ends with
     // the expert's last valid row: lanes that would load tokens past it get zeros and cause no
-    // traffic. Tiles of 32 tokens with no valid token are skipped altogether.
+    // traffic. Tiles of 32 tokens with no valid token are skipped altogether. When K is not a
+    // multiple of 64, the lanes that hold vectors past the end of a row in the last step are sent
+    // out of range there the same way (both operands: a zero times a stray NaN would not be zero).
     const int live = rows - t0;  // valid tokens of this block, > 0
-    const int row_bytes = H * 2;
+    const int row_bytes = K * 2;
     const __amdgpu_buffer_rsrc_t wbuf = __builtin_amdgcn_make_buffer_rsrc(
-        (void*)(weights + ((size_t)le * H + nw) * row_vecs), 0, 32 * row_bytes, BUFFER_RAW_32BIT);
+        (void*)(weights + ((size_t)le * N + nw) * row_vecs), 0, 32 * row_bytes, BUFFER_RAW_32BIT);
     const __amdgpu_buffer_rsrc_t xbuf = __builtin_amdgcn_make_buffer_rsrc(
         (void*)(expert_x + ((size_t)le * max_recv + t0) * row_vecs), 0, min(live, TOK) * row_bytes, BUFFER_RAW_32BIT);
-    int woff[4], wslot[4], xoff[TJ];
+    constexpr int OUT_OF_RANGE = 0x40000000;
+    int woff[4], wslot[4], xoff[TJ], wpast[2];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      const int row = sub + 8 * i;
-      woff[i] = row * row_bytes + (slot ^ ((row >> 1) & 7)) * 16;
+      const int row = sub + 8 * i, vec = slot ^ ((row >> 1) & 7);
+      woff[i] = row * row_bytes + vec * 16;
       wslot[i] = row * 8 + slot;
+      if (i < 2) wpast[i] = vec >= tail_vecs ? OUT_OF_RANGE : 0;  // (loads i and i + 2 take the same vector)
     }
     const int xrow = tid >> 3, xvec = slot ^ ((xrow >> 1) & 7);  // (32*i does not change bits 1..3)
+    const int xpast = xvec >= tail_vecs ? OUT_OF_RANGE : 0;
 #pragma unroll
     for (int i = 0; i < TJ; ++i) xoff[i] = (xrow + 32 * i) * row_bytes + xvec * 16;
 
     f32x16 acc[TJ] = {};
     b128 wv[D][4], xv[D][TJ];
     auto load_w = [&](int set, int step) {
-      const int k = min(step, steps - 1) * (GEMM_KSTEP * 2);  // past the end: the last step again, unused
+      const int at = min(step, steps - 1);  // past the end: the last step again, unused
+      const bool last = at == steps - 1;
 #pragma unroll
-      for (int i = 0; i < 4; ++i) wv[set][i] = __builtin_amdgcn_raw_buffer_load_b128(wbuf, woff[i], k, 0);
+      for (int i = 0; i < 4; ++i)
+        wv[set][i] = __builtin_amdgcn_raw_buffer_load_b128(wbuf, woff[i] + (last ? wpast[i & 1] : 0),
+                                                           at * (GEMM_KSTEP * 2), 0);
     };
     auto load_x = [&](int set, int step) {
-      const int k = min(step, steps - 1) * (GEMM_KSTEP * 2);
+      const int at = min(step, steps - 1);
+      const bool last = at == steps - 1;
 #pragma unroll
-      for (int i = 0; i < TJ; ++i) xv[set][i] = __builtin_amdgcn_raw_buffer_load_b128(xbuf, xoff[i], k, 0);
+      for (int i = 0; i < TJ; ++i)
+        xv[set][i] = __builtin_amdgcn_raw_buffer_load_b128(xbuf, xoff[i] + (last ? xpast : 0),
+                                                           at * (GEMM_KSTEP * 2), 0);
     };
     auto park_x = [&](int set) {
 #pragma unroll
@@ -1761,18 +1776,32 @@ __global__ __launch_bounds__(BLOCK, TJ <= 2 ? MOE_A2A_GEMM_OCC : 2) void expert_
     for (int u = 0; u < D - 1; ++u)
       if (at + u < steps) step(u, at + u);
 
-    // D[n][token] of a 32x32 tile: this lane holds token r and output columns g*8 + kb*4 + 0..3, g < 4
+    // D[n][token] of a 32x32 tile: this lane holds token r and output columns g*8 + kb*4 + 0..3, g < 4.
+    // With a bias the sum is rounded to the 16-bit type first and the bias added to that, as
+    // `matmul(x, w.T) + bias` on 16-bit tensors does (gemm-rs/reference.py:54-57).
     if (cols_valid) {
+      uint32_t bias2[4][2] = {};
+      if (bias) {
+#pragma unroll
+        for (int g = 0; g < 4; ++g) __builtin_memcpy(bias2[g], bias + (size_t)le * N + n0 + kb * 4 + g * 8, 8);
+      }
 #pragma unroll
       for (int j = 0; j < TJ; ++j) {
         const int token = t0 + j * 32 + r;
         if (token < rows) {
-          uint16_t* out = expert_y + ((size_t)le * max_recv + token) * H + n0 + kb * 4;
+          uint16_t* out = expert_y + ((size_t)le * max_recv + token) * N + n0 + kb * 4;
 #pragma unroll
           for (int g = 0; g < 4; ++g) {
             const f32x16& c = acc[j];
             uint32_t two[2] = {Pair16<DT>::canonical(Pair16<DT>::round(c[g * 4 + 0], c[g * 4 + 1])),
                                Pair16<DT>::canonical(Pair16<DT>::round(c[g * 4 + 2], c[g * 4 + 3]))};
+            if (bias) {
+#pragma unroll
+              for (int h = 0; h < 2; ++h)
+                two[h] = Pair16<DT>::canonical(Pair16<DT>::round(
+                    __fadd_rn(Pair16<DT>::lo(two[h]), Pair16<DT>::lo(bias2[g][h])),
+                    __fadd_rn(Pair16<DT>::hi(two[h]), Pair16<DT>::hi(bias2[g][h]))));
+            }
             __builtin_memcpy(out + g * 8, two, 8);
           }
         }
@@ -2264,30 +2293,33 @@ int moe_a2a_expert_scale(const moe_a2a_shape* s, const void* expert_x,
 }
 
 #ifndef MOE_A2A_GEMM_ROWS_FOR_128
-#define MOE_A2A_GEMM_ROWS_FOR_128 48  // rows per expert (mean, from the hint) above which blocks hold 128 tokens
+#define MOE_A2A_GEMM_ROWS_FOR_128 48  // rows per group (mean, from the hint) above which blocks hold 128 tokens
 #endif
 
-int moe_a2a_expert_gemm(const moe_a2a_shape* s, const void* expert_x,
-                        const int32_t* expert_num_tokens, int32_t rows_hint, const void* weights,
-                        int32_t dtype, void* expert_y, void* stream) {
-  if (!shape_ok(s) || rows_hint < 0 || !expert_x || !expert_num_tokens || !weights || !expert_y)
-    return MOE_A2A_EINVAL;
+}  // extern "C"
+
+namespace {
+
+// y[g, :rows(g), :] = x[g, :rows(g), :] @ w[g]^T (+ bias[g]) for `groups` groups of at most max_rows
+// rows; rows_of_group null means max_rows rows in every group.
+int launch_grouped_gemm(const void* x, const int32_t* rows_of_group, const void* w, const void* bias,
+                        void* y, int groups, long long max_rows, long long rows_hint, int N, int K,
+                        int dtype, hipStream_t st) {
   if (dtype != MOE_A2A_F16 && dtype != MOE_A2A_BF16) return MOE_A2A_EINVAL;
-  if (s->hidden_dim % GEMM_KSTEP != 0) return MOE_A2A_EINVAL;  // whole steps of the input
-  if (!all_aligned(16, expert_x, weights, expert_y)) return MOE_A2A_EALIGN;
-  const int nle = s->num_experts / s->world_size;
-  const long long max_recv = (long long)s->max_num_tokens * s->world_size;
-  const int col_tiles = (s->hidden_dim + GEMM_COLS - 1) / GEMM_COLS;
-  const int tj = (long long)rows_hint > (long long)MOE_A2A_GEMM_ROWS_FOR_128 * nle ? 4 : 2;
-  // every expert can end in a partly filled block of tokens; the kernel strides over what the hint misses
-  const long long row_blocks = (long long)rows_hint / (tj * 32) + nle;
-  if ((max_recv / 64 + 1) * nle * col_tiles > INT_MAX / 2) return MOE_A2A_EINVAL;
+  if (N % 32 != 0 || K % 8 != 0) return MOE_A2A_EINVAL;  // whole wave tiles of columns, whole 16-byte vectors
+  if (!all_aligned(16, x, w, y) || !all_aligned(8, bias)) return MOE_A2A_EALIGN;
+  // per-lane byte offsets inside a block of tokens and inside a wave's 32 weight rows are 32-bit
+  if ((long long)K * 2 * 128 >= (1 << 30) || max_rows > INT_MAX / 2) return MOE_A2A_EINVAL;
+  const int col_tiles = (N + GEMM_COLS - 1) / GEMM_COLS;
+  const int tj = rows_hint > (long long)MOE_A2A_GEMM_ROWS_FOR_128 * groups ? 4 : 2;
+  // every group can end in a partly filled block of tokens; the kernel strides over what the hint misses
+  const long long row_blocks = rows_hint / (tj * 32) + groups;
+  if ((max_rows / 64 + 1) * groups * col_tiles > INT_MAX / 2) return MOE_A2A_EINVAL;
   const int grid = mover_blocks(row_blocks * col_tiles);
-  hipStream_t st = (hipStream_t)stream;
-#define LAUNCH_G(DT, TJ)                                                                         \
-  expert_gemm_kernel<DT, TJ><<<grid, BLOCK, 0, st>>>((const b128*)expert_x, expert_num_tokens,   \
-                                                     (const b128*)weights, (uint16_t*)expert_y,  \
-                                                     nle, (int)max_recv, s->hidden_dim, col_tiles)
+#define LAUNCH_G(DT, TJ)                                                                          \
+  expert_gemm_kernel<DT, TJ><<<grid, BLOCK, 0, st>>>((const b128*)x, rows_of_group, (const b128*)w, \
+                                                     (const uint16_t*)bias, (uint16_t*)y, groups,  \
+                                                     (int)max_rows, N, K, col_tiles)
   if (dtype == MOE_A2A_BF16) {
     if (tj == 2) LAUNCH_G(MOE_A2A_BF16, 2);
     else LAUNCH_G(MOE_A2A_BF16, 4);
@@ -2297,6 +2329,29 @@ int moe_a2a_expert_gemm(const moe_a2a_shape* s, const void* expert_x,
   }
 #undef LAUNCH_G
   return launch_status();
+}
+
+}  // namespace
+
+extern "C" {
+
+int moe_a2a_expert_gemm(const moe_a2a_shape* s, const void* expert_x,
+                        const int32_t* expert_num_tokens, int32_t rows_hint, const void* weights,
+                        int32_t dtype, void* expert_y, void* stream) {
+  if (!shape_ok(s) || rows_hint < 0 || !expert_x || !expert_num_tokens || !weights || !expert_y)
+    return MOE_A2A_EINVAL;
+  const int nle = s->num_experts / s->world_size;
+  const long long max_recv = (long long)s->max_num_tokens * s->world_size;
+  return launch_grouped_gemm(expert_x, expert_num_tokens, weights, nullptr, expert_y, nle, max_recv,
+                             rows_hint, s->hidden_dim, s->hidden_dim, dtype, (hipStream_t)stream);
+}
+
+int moe_a2a_linear(const void* input, const void* weight, const void* bias, int32_t m, int32_t n,
+                   int32_t k, int32_t dtype, void* output, void* stream) {
+  if (m < 0 || n < 1 || k < 1 || !weight || (m > 0 && (!input || !output))) return MOE_A2A_EINVAL;
+  if (m == 0) return MOE_A2A_OK;
+  return launch_grouped_gemm(input, nullptr, weight, bias, output, 1, m, m, n, k, dtype,
+                             (hipStream_t)stream);
 }
 
 int moe_a2a_exchange_local(int32_t world_size, int32_t hidden_dim, const void* send_buf,

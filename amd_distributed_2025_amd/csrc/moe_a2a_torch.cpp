@@ -199,6 +199,26 @@ void a2a_expert_gemm(std::vector<int64_t> shape, torch::Tensor expert_x, torch::
          "moe_a2a_expert_gemm");
 }
 
+void a2a_linear(torch::Tensor input, torch::Tensor weight, c10::optional<torch::Tensor> bias, torch::Tensor output,
+                int64_t stream) {
+  const auto dt = rows_type(input, "input");
+  TORCH_CHECK(input.dim() == 2 && weight.dim() == 2 && output.dim() == 2, "input, weight and output must be 2-D");
+  const int64_t m = input.size(0), k = input.size(1), n = weight.size(0);
+  need(input, "input", dt, m * k);
+  need(weight, "weight", dt, n * k, &input);
+  need(output, "output", dt, m * n, &input);
+  TORCH_CHECK(weight.size(1) == k, "weight must be [n, k] with k = input.size(1)");
+  TORCH_CHECK(output.size(0) == m && output.size(1) == n, "output must be [m, n]");
+  const void* b = nullptr;
+  if (bias.has_value()) {
+    need(*bias, "bias", dt, n, &input);
+    b = bias->data_ptr();
+  }
+  status(moe_a2a_linear(input.data_ptr(), weight.data_ptr(), b, to_i32(m, "m"), to_i32(n, "n"), to_i32(k, "k"),
+                        dtype_code(dt), output.data_ptr(), stream_of(stream)),
+         "moe_a2a_linear");
+}
+
 void a2a_exchange_local(int64_t world_size, int64_t hidden_dim, torch::Tensor send_buf, torch::Tensor send_meta,
                         torch::Tensor send_counts, int64_t dst_rank, torch::Tensor recv_buf,
                         torch::Tensor recv_meta, torch::Tensor recv_counts, int64_t src_rank, int64_t rows_hint,

@@ -1,0 +1,74 @@
+"""The one-GPU part of the reference's gemm-rs task: `input @ weight.T (+ bias)`.
+
+The reference's `ref_kernel` (gemm-rs/reference.py:36-60) multiplies this rank's
+[M, local_K] slice of the activations with its [N, local_K] slice of the weight,
+adds the bias, and reduce-scatters the [M, N] partial products over the ranks.
+`local_product` is everything up to the reduce-scatter, on the matrix cores of
+one MI355X through `moe_a2a_linear`; the reduce-scatter is an exchange between
+GPUs and is not part of this package. `custom_kernel` therefore serves a job of
+one rank (where the reduce-scatter is the identity) and refuses larger ones.
+
+`generate_input` restates gemm-rs/reference.py:5-33 (uniform values in
+[-0.01, 0.01), bias drawn from the job seed so that all ranks share it).
+"""
+from __future__ import annotations
+
+from typing import Optional, Tuple
+
+import torch
+
+from . import _binding
+
+input_t = Tuple[torch.Tensor, torch.Tensor, Optional[torch.Tensor]]
+
+
+def generate_input(rank: int, world_size: int, m: int, n: int, k: int, has_bias: bool, seed: int,
+                   device=None) -> input_t:
+    device = torch.device(device if device is not None else f"cuda:{rank}")
+    gen = torch.Generator(device=device)
+    gen.manual_seed(seed + rank)
+    if m % world_size or k % world_size:
+        raise ValueError("m and k must be divisible by world_size")
+    local_k = k // world_size
+    inp = (torch.rand((m, local_k), dtype=torch.bfloat16, device=device, generator=gen) * 2 - 1) * 0.01
+    weight = (torch.rand((n, local_k), dtype=torch.bfloat16, device=device, generator=gen) * 2 - 1) * 0.01
+    bias = None
+    if has_bias:
+        gen.manual_seed(seed)
+        bias = (torch.rand((n,), dtype=torch.bfloat16, device=device, generator=gen) * 2 - 1) * 0.01
+    return inp, weight, bias
+
+
+def local_product(data: input_t, out: Optional[torch.Tensor] = None, binding: str = "ctypes") -> torch.Tensor:
+    """`matmul(input, weight.T)` rounded to the 16-bit type, then `+ bias` rounded again
+    (gemm-rs/reference.py:54-57), as one launch. Returns [M, N]."""
+    inp, weight, bias = data
+    if inp.dim() != 2 or weight.dim() != 2 or inp.shape[1] != weight.shape[1]:
+        raise ValueError(f"input [M, K] and weight [N, K] expected, got {tuple(inp.shape)} and {tuple(weight.shape)}")
+    if inp.dtype not in (torch.float16, torch.bfloat16):
+        raise TypeError(f"input: expected float16 or bfloat16, got {inp.dtype}")
+    if not inp.is_cuda:
+        raise ValueError("input: expected a GPU tensor (there is no CPU path)")
+    tensors = [("weight", weight)] + ([("bias", bias)] if bias is not None else [])
+    for what, t in [("input", inp)] + tensors:
+        if t.dtype != inp.dtype or t.device != inp.device or not t.is_contiguous():
+            raise ValueError(f"{what}: must be contiguous, {inp.dtype}, on {inp.device}")
+    m, n = inp.shape[0], weight.shape[0]
+    if bias is not None and tuple(bias.shape) != (n,):
+        raise ValueError(f"bias must be [{n}], got {tuple(bias.shape)}")
+    if out is None:
+        out = torch.empty((m, n), dtype=inp.dtype, device=inp.device)
+    elif tuple(out.shape) != (m, n) or out.dtype != inp.dtype or out.device != inp.device or not out.is_contiguous():
+        raise ValueError(f"out must be a contiguous [{m}, {n}] {inp.dtype} tensor on {inp.device}")
+    stream = torch.cuda.current_stream(inp.device).cuda_stream
+    _binding.get(binding).linear(inp, weight, bias, out, stream)
+    return out
+
+
+def custom_kernel(data: input_t) -> torch.Tensor:
+    """The reference's entry point (gemm-rs/submission.py:9-29) for a job of one rank."""
+    world_size = torch.distributed.get_world_size() if torch.distributed.is_initialized() else 1
+    if world_size != 1:
+        raise NotImplementedError("the reduce-scatter over several GPUs is outside this package; "
+                                  "local_product() gives this rank's [M, N] partial product")
+    return local_product(data)

@@ -274,19 +274,36 @@ int moe_a2a_expert_scale(const moe_a2a_shape* shape, const void* expert_x,
  *   dtype      MOE_A2A_F16 or MOE_A2A_BF16: element type of all three
  *   expert_y   [nle, max_recv, H] out; rows at or past expert_num_tokens[le] are
  *              not written
- * Rows are processed in blocks of 128 found from the device-side counts, so the
- * work follows the rows, not the experts. Limits: hidden_dim a multiple of 64,
- * all three buffers 16-byte aligned, nle <= 4096 (MOE_A2A_EINVAL / EALIGN).
+ * Rows are processed in blocks of 64 or 128 tokens found from the device-side
+ * counts, so the work follows the rows, not the experts. Limits: hidden_dim a
+ * multiple of 32, all three buffers 16-byte aligned (MOE_A2A_EINVAL / EALIGN).
  * Sums are formed in float32 in the order of the matrix unit, which is not the
- * order of a CPU matmul: results agree with a float32 reference to within one
- * unit in the last place of the 16-bit type plus the float32 summation error,
- * and exactly when every sum has at most one nonzero term per 16 inputs that is
- * exactly representable (identity and signed permutation weights).
+ * order of a CPU matmul: results lie within what float32 accumulation in any
+ * order plus one rounding allows around the exact product, and are exact when
+ * every order gives the same float32 sum (identity and signed permutation
+ * weights, small integers).
  */
 int moe_a2a_expert_gemm(const moe_a2a_shape* shape, const void* expert_x,
                         const int32_t* expert_num_tokens, int32_t rows_hint,
                         const void* weights, int32_t dtype, void* expert_y,
                         void* stream);
+
+/*
+ * output[m, n] = input[m, k] @ weight[n, k]^T (+ bias[n]): the product one rank
+ * computes in the reference's gemm-rs task before the reduce-scatter
+ * (gemm-rs/reference.py:54-57: `torch.matmul(input, weight.T)`, then
+ * `output + bias`). Same kernel as moe_a2a_expert_gemm with one group of m rows.
+ * All tensors are of the 16-bit type `dtype` (MOE_A2A_F16 / MOE_A2A_BF16), row-major,
+ * k contiguous in input and weight. Accumulation is float32 with one rounding
+ * to the 16-bit type; a bias is then added to that rounded value and the sum
+ * rounded again, which is what the two torch statements do. bias may be NULL.
+ * Limits: n a multiple of 32, k a multiple of 8, input / weight / output 16-byte
+ * and bias 8-byte aligned (MOE_A2A_EINVAL / EALIGN). m == 0 is a no-op.
+ * The reduce-scatter that follows in the reference (gemm-rs/reference.py:58-59)
+ * is an exchange between GPUs and not part of this library.
+ */
+int moe_a2a_linear(const void* input, const void* weight, const void* bias, int32_t m,
+                   int32_t n, int32_t k, int32_t dtype, void* output, void* stream);
 
 /*
  * Stand-in for one (source rank -> destination rank) leg of the exchange,

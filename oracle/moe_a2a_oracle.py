@@ -214,6 +214,27 @@ def expert_gemm_bound(rows: np.ndarray, weights: np.ndarray, dtype: str):
     return exact, u16 * (np.abs(exact) + sum_err) + sum_err + floor
 
 
+def linear(inp: np.ndarray, weight: np.ndarray, bias, dtype: str) -> np.ndarray:
+    """`torch.matmul(input, weight.T)` then `output + bias` on 16-bit tensors
+    (gemm-rs/reference.py:54-57): the product is rounded to the 16-bit type, the
+    bias is added to the rounded value in float32 and the sum rounded again."""
+    out = expert_gemm(inp, weight, dtype)
+    if bias is None:
+        return out
+    return f32_to_b16(b16_to_f32(out, dtype) + b16_to_f32(bias, dtype)[None, :], dtype)
+
+
+def linear_bound(inp: np.ndarray, weight: np.ndarray, bias, dtype: str):
+    """(exact, tol) for `linear`: the float64 value of input @ weight.T + bias and how far
+    from it the twice-rounded result can lie for any float32 summation order."""
+    exact, tol = expert_gemm_bound(inp, weight, dtype)
+    if bias is None:
+        return exact, tol
+    u16 = 2.0 ** -8 if dtype == "bf16" else 2.0 ** -11
+    total = exact + b16_to_f32(bias, dtype).astype(np.float64)[None, :]
+    return total, tol + (u16 + 2.0 ** -23) * (np.abs(total) + tol)
+
+
 # ----------------------------------------------------------------------------- combine
 
 

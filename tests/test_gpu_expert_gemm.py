@@ -50,7 +50,7 @@ def ragged_counts(rng, nle, max_recv, special):
 
 
 @pytest.mark.parametrize("dt", [torch.bfloat16, torch.float16], ids=["bf16", "fp16"])
-@pytest.mark.parametrize("W,nle,H,max_tokens", [(1, 1, 64, 16), (2, 3, 192, 80), (4, 8, 2048, 128), (8, 2, 7168, 40)])
+@pytest.mark.parametrize("W,nle,H,max_tokens", [(1, 1, 64, 16), (1, 2, 32, 8), (2, 3, 96, 40), (2, 3, 192, 80), (4, 8, 2048, 128), (8, 2, 7168, 40)])
 def test_signed_permutation_weights_move_columns_exactly(W, nle, H, max_tokens, dt):
     print(f"permutation W={W} nle={nle} H={H} T={max_tokens} {dt}", flush=True)
     rng = np.random.default_rng(H + nle)
@@ -78,7 +78,7 @@ def test_signed_permutation_weights_move_columns_exactly(W, nle, H, max_tokens, 
 
 
 @pytest.mark.parametrize("dt", [torch.bfloat16, torch.float16], ids=["bf16", "fp16"])
-@pytest.mark.parametrize("H", [128, 192])
+@pytest.mark.parametrize("H", [96, 128, 192])
 def test_small_integers_sum_exactly(H, dt):
     print(f"integers H={H} {dt}", flush=True)
     rng = np.random.default_rng(H)
@@ -183,9 +183,9 @@ def test_both_bindings_give_the_same_bits():
 
 
 def test_unsupported_shapes_raise():
-    a, cfg = rank_object(1, 1, 96, 4, torch.bfloat16)
-    ex = torch.zeros(1, 4, 96, dtype=torch.bfloat16, device=DEV)
-    w = torch.zeros(1, 96, 96, dtype=torch.bfloat16, device=DEV)
+    a, cfg = rank_object(1, 1, 80, 4, torch.bfloat16)  # not whole wave tiles of 32 columns
+    ex = torch.zeros(1, 4, 80, dtype=torch.bfloat16, device=DEV)
+    w = torch.zeros(1, 80, 80, dtype=torch.bfloat16, device=DEV)
     with pytest.raises(Exception, match="invalid|argument"):
         a.expert_gemm(ex, torch.tensor([4], dtype=torch.int32, device=DEV), w)
     with pytest.raises(ValueError, match="weights must be"):

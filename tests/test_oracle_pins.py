@@ -278,3 +278,64 @@ def test_combine_accumulates_onto_given_rows():
         t, k = int(meta[i, 2]), int(meta[i, 3])
         y[t] += rb[i].float() * torch.tensor(w[t, k])
     assert np.array_equal(got, y.view(torch.int16).numpy().view(np.uint16))
+
+
+# ----------------------------------------------------------------------------- matrix products
+
+def _b(t: torch.Tensor) -> np.ndarray:
+    return t.contiguous().view(torch.int16).numpy().view(np.uint16)
+
+
+@pytest.mark.parametrize("name,tdt", [("bf16", torch.bfloat16), ("fp16", torch.float16)])
+def test_gemm_oracle_on_inputs_where_every_summation_order_agrees(name, tdt):
+    # small integers: a brute-force integer loop is the answer, whatever the order of the sum
+    x = RNG.integers(-2, 3, (7, 24))
+    w = RNG.integers(-2, 3, (5, 24))
+    want = np.array([[sum(int(x[i, k]) * int(w[j, k]) for k in range(24)) for j in range(5)] for i in range(7)])
+    got = orc.expert_gemm(_b(torch.from_numpy(x).to(tdt)), _b(torch.from_numpy(w).to(tdt)), name)
+    assert np.array_equal(orc.b16_to_f32(got, name), want.astype(np.float32))
+    # a signed permutation as weights moves columns: out[:, j] = sign[j] * x[:, perm[j]] (not its transpose)
+    perm, sign = RNG.permutation(24), RNG.choice([-1.0, 1.0], 24)
+    pw = np.zeros((24, 24), np.float32)
+    pw[np.arange(24), perm] = sign
+    rows = RNG.integers(0, 1 << 15, (9, 24), dtype=np.uint16)  # positive finite-or-not patterns
+    rows[~np.isfinite(orc.b16_to_f32(rows, name))] = 0x3C00
+    got = orc.expert_gemm(rows, _b(torch.from_numpy(pw).to(tdt)), name)
+    want = np.where(sign[None, :] < 0, rows[:, perm] ^ 0x8000, rows[:, perm])
+    zero = (want & 0x7FFF) == 0
+    assert np.array_equal(got[~zero], want[~zero])
+
+
+@pytest.mark.parametrize("name,tdt", [("bf16", torch.bfloat16), ("fp16", torch.float16)])
+def test_linear_oracle_is_the_torch_expression(name, tdt):
+    # gemm-rs/reference.py:54-57 on the CPU, on integers (exact in any order) ...
+    x = torch.from_numpy(RNG.integers(-3, 4, (11, 40))).to(tdt)
+    w = torch.from_numpy(RNG.integers(-3, 4, (6, 40))).to(tdt)
+    b = torch.from_numpy(RNG.integers(-9, 10, 6)).to(tdt)
+    assert np.array_equal(orc.linear(_b(x), _b(w), _b(b), name), _b(torch.matmul(x, w.T) + b))
+    assert np.array_equal(orc.linear(_b(x), _b(w), None, name), _b(torch.matmul(x, w.T)))
+    # ... and where the two roundings show: the product is rounded before the bias is added
+    u = 2.0 ** -8 if name == "bf16" else 2.0 ** -11
+    x = torch.tensor([[1.0, u]], dtype=tdt)
+    w = torch.ones(3, 2, dtype=tdt)
+    b = torch.full((3,), 2 * u, dtype=tdt)
+    want = torch.matmul(x, w.T) + b
+    assert float(want[0, 0]) == 1.0 + 2 * u  # (1 + u rounds to 1 first; added unrounded it would reach 1 + 4u)
+    assert np.array_equal(orc.linear(_b(x), _b(w), _b(b), name), _b(want))
+
+
+def test_gemm_bound_holds_for_torch_and_catches_a_dropped_term():
+    x = torch.randn(33, 512, generator=torch.Generator().manual_seed(1)).to(torch.bfloat16)
+    w = (torch.randn(48, 512, generator=torch.Generator().manual_seed(2)) / 512 ** 0.5).to(torch.bfloat16)
+    exact, tol = orc.expert_gemm_bound(_b(x), _b(w), "bf16")
+    for got in (orc.expert_gemm(_b(x), _b(w), "bf16"), _b(torch.matmul(x, w.T)),
+                _b((x.float() @ w.float().T).to(torch.bfloat16))):
+        assert (np.abs(orc.b16_to_f32(got, "bf16").astype(np.float64) - exact) <= tol).all()
+    # one input left out of every sum: most results leave the bound
+    short = _b((x[:, :-1].float() @ w[:, :-1].float().T).to(torch.bfloat16))
+    assert (np.abs(orc.b16_to_f32(short, "bf16").astype(np.float64) - exact) > tol).mean() > 0.5
+    # operands swapped (w @ x.T, transposed back) is the same product; a transposed weight is not
+    sq = (torch.randn(512, 512, generator=torch.Generator().manual_seed(3)) / 512 ** 0.5).to(torch.bfloat16)
+    exact, tol = orc.expert_gemm_bound(_b(x), _b(sq), "bf16")
+    wrong = _b((x.float() @ sq.float()).to(torch.bfloat16))
+    assert (np.abs(orc.b16_to_f32(wrong, "bf16").astype(np.float64) - exact) > tol).mean() > 0.5
