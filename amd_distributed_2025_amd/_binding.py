@@ -50,11 +50,17 @@ class CtypesBinding:
                   _ptr(rank_offsets), _ptr(expert_counts), _ptr(dst_slot), _ptr(src_entry), C.c_void_p(stream))
 
     def dispatch_recv(self, shape, recv_buf, recv_meta, recv_counts, rows_hint, expert_num_tokens, expert_x,
-                      expert_meta, send_back_plan, stream):
+                      expert_meta, send_back_plan, stream, row_position=None):
         capacity = _rows(recv_buf, recv_meta, shape.hidden_dim)
-        _lib.call("moe_a2a_dispatch_recv", C.byref(shape), _ptr(recv_buf), _ptr(recv_meta), _ptr(recv_counts),
-                  min(rows_hint, capacity), capacity, _ptr(expert_num_tokens), _ptr(expert_x), _ptr(expert_meta),
-                  _ptr(send_back_plan), C.c_void_p(stream))
+        args = (C.byref(shape), _ptr(recv_buf), _ptr(recv_meta), _ptr(recv_counts),
+                min(rows_hint, capacity), capacity, _ptr(expert_num_tokens), _ptr(expert_x), _ptr(expert_meta),
+                _ptr(send_back_plan))
+        if row_position is None:
+            _lib.call("moe_a2a_dispatch_recv", *args, C.c_void_p(stream))
+        else:  # long streams: positions from a planning launch
+            if row_position.numel() < capacity:
+                raise ValueError("row_position must hold one int per row of the receive buffers")
+            _lib.call("moe_a2a_dispatch_recv_long", *args, _ptr(row_position), C.c_void_p(stream))
 
     def combine_send(self, shape, expert_y, expert_meta, expert_num_tokens, rows_hint, send_buf, send_meta,
                      send_counts, send_back_plan, stream):
@@ -64,11 +70,17 @@ class CtypesBinding:
                   _ptr(send_counts), _ptr(send_back_plan), C.c_void_p(stream))
 
     def combine_recv(self, shape, recv_buf, recv_meta, recv_counts, rows_hint, weights, num_tokens, out_tokens,
-                     accumulate, stream):
+                     accumulate, stream, entry_row=None):
         capacity = _rows(recv_buf, recv_meta, shape.hidden_dim)
-        _lib.call("moe_a2a_combine_recv", C.byref(shape), _ptr(recv_buf), _ptr(recv_meta), _ptr(recv_counts),
-                  min(rows_hint, capacity), capacity, _ptr(weights), num_tokens, _ptr(out_tokens),
-                  int(bool(accumulate)), _DT[out_tokens.dtype], C.c_void_p(stream))
+        args = (C.byref(shape), _ptr(recv_buf), _ptr(recv_meta), _ptr(recv_counts),
+                min(rows_hint, capacity), capacity, _ptr(weights), num_tokens, _ptr(out_tokens),
+                int(bool(accumulate)), _DT[out_tokens.dtype])
+        if entry_row is None:
+            _lib.call("moe_a2a_combine_recv", *args, C.c_void_p(stream))
+        else:  # long streams: rows looked up in a (token, k) -> row table
+            if entry_row.numel() < num_tokens * shape.experts_per_token:
+                raise ValueError("entry_row must hold num_tokens * experts_per_token ints")
+            _lib.call("moe_a2a_combine_recv_long", *args, _ptr(entry_row), C.c_void_p(stream))
 
     def expert_scale(self, shape, expert_x, expert_num_tokens, rows_hint, expert_y, stream):
         _lib.call("moe_a2a_expert_scale", C.byref(shape), _ptr(expert_x), _ptr(expert_num_tokens), rows_hint,
@@ -116,9 +128,9 @@ class ExtBinding:
                               dst_slot, src_entry, stream)
 
     def dispatch_recv(self, shape, recv_buf, recv_meta, recv_counts, rows_hint, expert_num_tokens, expert_x,
-                      expert_meta, send_back_plan, stream):
+                      expert_meta, send_back_plan, stream, row_position=None):
         self._m.a2a_dispatch_recv(self._shape(shape), recv_buf, recv_meta, recv_counts, rows_hint,
-                                  expert_num_tokens, expert_x, expert_meta, send_back_plan, stream)
+                                  expert_num_tokens, expert_x, expert_meta, send_back_plan, row_position, stream)
 
     def combine_send(self, shape, expert_y, expert_meta, expert_num_tokens, rows_hint, send_buf, send_meta,
                      send_counts, send_back_plan, stream):
@@ -126,9 +138,9 @@ class ExtBinding:
                                  send_buf, send_meta, send_counts, send_back_plan, stream)
 
     def combine_recv(self, shape, recv_buf, recv_meta, recv_counts, rows_hint, weights, num_tokens, out_tokens,
-                     accumulate, stream):
+                     accumulate, stream, entry_row=None):
         self._m.a2a_combine_recv(self._shape(shape), recv_buf, recv_meta, recv_counts, rows_hint, weights,
-                                 num_tokens, out_tokens, bool(accumulate), stream)
+                                 num_tokens, out_tokens, bool(accumulate), entry_row, stream)
 
     def expert_scale(self, shape, expert_x, expert_num_tokens, rows_hint, expert_y, stream):
         self._m.a2a_expert_scale(self._shape(shape), expert_x, expert_num_tokens, rows_hint, expert_y, stream)

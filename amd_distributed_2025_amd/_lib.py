@@ -41,9 +41,11 @@ SIGNATURES = {
     "moe_a2a_dispatch_send": [_SP, _P, _P, _I, _P, _P, _P, _P, _P],
     "moe_a2a_plan_send": [_SP, _P, _I, _P, _P, _P, _P, _P, _P],
     "moe_a2a_dispatch_recv": [_SP, _P, _P, _P, _I, _I, _P, _P, _P, _P, _P],
+    "moe_a2a_dispatch_recv_long": [_SP, _P, _P, _P, _I, _I, _P, _P, _P, _P, _P, _P],
     "moe_a2a_dispatch_recv_static": [_SP, _P, _P, _P, _I, _I, _P, _P, _P, C.POINTER(C.c_void_p), _P],
     "moe_a2a_combine_send": [_SP, _P, _P, _P, _I, _I, _P, _P, _P, _P, _P],
     "moe_a2a_combine_recv": [_SP, _P, _P, _P, _I, _I, _P, _I, _P, _I, _I, _P],
+    "moe_a2a_combine_recv_long": [_SP, _P, _P, _P, _I, _I, _P, _I, _P, _I, _I, _P, _P],
     "moe_a2a_expert_scale": [_SP, _P, _P, _I, _I, _I, _P, _P],
     "moe_a2a_expert_gemm": [_SP, _P, _P, _I, _P, _I, _P, _P],
     "moe_a2a_linear": [_P, _P, _P, _I, _I, _I, _I, _P, _P],

@@ -32,6 +32,12 @@ from . import _binding, _lib
 from .task import MoEConfig, RankTestData
 
 META_DIM = 5
+# Streams of more rows than this take the entry points that rank in a planning launch of their
+# own (moe_a2a_dispatch_recv_long, moe_a2a_combine_recv_long); shorter ones the one-launch
+# entry points, whose movers rank by scanning. Results are the same; the second launch costs
+# 5-7 us, which the combine earns back from about 4096 rows and the dispatch (whose scans hide
+# behind its payload for longer) from about 12288 (measured at hidden_dim 7168).
+LONG_STREAM_ROWS = {"dispatch": 12288, "combine": 4096}
 
 
 def _stream(device) -> int:
@@ -76,6 +82,7 @@ class HIPAllToAll:
         # it when it is handed the very tensors that dispatch_recv returned
         self.reuse_placement = reuse_placement
         self._planned_for = None
+        self.long_stream_rows = None  # an int overrides both thresholds of LONG_STREAM_ROWS
 
     # ------------------------------------------------------------------ workspace
 
@@ -151,8 +158,9 @@ class HIPAllToAll:
         ex = self._buf("expert_x", (nle, self.max_recv, cfg.hidden_dim), cfg.in_dtype)
         em = self._buf("expert_meta", (nle, self.max_recv, META_DIM), torch.int32)
         plan = self._buf("send_back_plan", (2 * cfg.num_experts,), torch.int32) if self.reuse_placement else None
+        pos = self._buf("row_position", (capacity,), torch.int32) if hint > self._long_from("dispatch") else None
         self.binding.dispatch_recv(self.shape, recv_buf, recv_meta, recv_counts, hint, num, ex, em, plan,
-                                   _stream(self.device))
+                                   _stream(self.device), pos)
         self._planned_for = None if plan is None else (em.data_ptr(), num.data_ptr())
         self._rows_in_hint = hint
         return num, ex, em
@@ -225,9 +233,15 @@ class HIPAllToAll:
             raise ValueError("combine: out_tokens must hold num_tokens rows of hidden_dim")
         capacity = min(ret_buf.shape[0], ret_meta.shape[0])
         hint = min(capacity, T * cfg.experts_per_token)
+        table = None
+        if hint > self._long_from("combine"):
+            table = self._buf("entry_row", (cfg.max_num_tokens * cfg.experts_per_token,), torch.int32)
         self.binding.combine_recv(self.shape, ret_buf, ret_meta, ret_counts, hint, weights, T, out_tokens,
-                                  accumulate, _stream(self.device))
+                                  accumulate, _stream(self.device), table)
         return out_tokens
+
+    def _long_from(self, phase: str) -> int:
+        return LONG_STREAM_ROWS[phase] if self.long_stream_rows is None else self.long_stream_rows
 
     def _default_rows_in(self, rows_hint):
         if rows_hint is not None:
@@ -343,10 +357,14 @@ class LocalWorld:
     device copies (stand-in for all2all/reference.py:91,107-119,185,210-222)."""
 
     def __init__(self, cfg: MoEConfig, world_size: int, device=None, exact_hints: bool = True,
-                 reuse_placement: bool = True, binding: str = "ctypes"):
+                 reuse_placement: bool = True, binding: str = "ctypes",
+                 long_stream_rows: Optional[int] = None):
         self.cfg, self.world_size = cfg, world_size
         self.ranks = [HIPAllToAll(cfg, r, world_size, device=device, reuse_placement=reuse_placement,
                                   binding=binding) for r in range(world_size)]
+        if long_stream_rows is not None:  # (0: every receive half takes the long-stream entry points)
+            for a in self.ranks:
+                a.long_stream_rows = long_stream_rows
         self.device = self.ranks[0].device
         # True: read the counts back to size every launch exactly (synchronises the host);
         # False: size for the worst case; "last": reuse what the previous run read back, for

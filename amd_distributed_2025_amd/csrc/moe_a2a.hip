@@ -24,6 +24,7 @@
 #include <hip/hip_fp16.h>
 #include <stdint.h>
 #include <limits.h>
+#include <algorithm>
 #include <mutex>
 #include <type_traits>
 
@@ -793,12 +794,92 @@ __global__ __launch_bounds__(PLAN_BLOCK) void plan_send_kernel(
 
 constexpr int PLAN_INTS = 2;  // ints per (local expert, source rank) of the send-back plan
 
-template <typename V, int NVW, bool PLAN>
+// Long streams. The movers below rank a row by counting the keys ahead of it, and every
+// workgroup of four rows repeats that pass: the key loads grow with the square of the row count
+// (at 8192 rows they are two thirds of the payload). For long streams the positions are worked
+// out by a launch of their own, one workgroup of 1024 lanes per tile of 1024 rows: an LDS
+// histogram (atomics; the order of the adds does not matter) of the experts of all rows ahead of
+// the tile, then inside the tile a row's rank among the earlier lanes of its wave with the same
+// expert from one ballot per expert present in the wave, the waves ordered by a prefix over
+// their per-expert counts. row_pos[i] = #{rows before i with the same local expert}, which is
+// the slot the reference's running counter hands out (all2all/reference.py:140-146). The movers
+// then read one int per row instead of scanning.
+constexpr int RPLAN_BLOCK = 1024;
+constexpr int RPLAN_WAVES = RPLAN_BLOCK / 64;
+constexpr int RPLAN_MAX_EXPERTS = 256;  // local experts with a counter per wave in LDS
+
+__global__ __launch_bounds__(RPLAN_BLOCK) void plan_recv_kernel(
+    const int* __restrict__ recv_meta, const int* __restrict__ recv_counts, int W, int hint_rows,
+    int capacity_rows, int nle, uint32_t magic, int* __restrict__ row_pos) {
+  __shared__ int ahead[RPLAN_MAX_EXPERTS];                  // rows of each expert before the tile
+  __shared__ int in_wave[RPLAN_WAVES][RPLAN_MAX_EXPERTS];   // rows of each expert in each wave of the tile
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const unsigned long long lanes_below = lane == 0 ? 0ull : (~0ull >> (64 - lane));
+  int R = -1;  // not known yet
+  auto rows = [&] { return min(sum_counts(recv_counts, W, capacity_rows), capacity_rows); };
+  for (int first = blockIdx.x * RPLAN_BLOCK;; first += gridDim.x * RPLAN_BLOCK) {
+    // A tile that lies wholly below the readable bound sends its loads off before the row
+    // count is known: the counts travel at the same time (one round trip instead of three).
+    const bool early = R < 0 && first + RPLAN_BLOCK <= hint_rows;
+    if (!early) {
+      if (R < 0) R = rows();
+      if (first >= R) break;
+    }
+    const int last = early ? first + RPLAN_BLOCK - 1 : R - 1;  // last row that may be read
+    const int i = first + tid;
+    const int mine = recv_meta[(size_t)min(i, last) * META];
+    int e2[SCAN_UNROLL];
+#pragma unroll
+    for (int u = 0; u < SCAN_UNROLL; ++u)
+      e2[u] = recv_meta[(size_t)min(tid + u * RPLAN_BLOCK, max(first - 1, 0)) * META];
+    for (int j = tid; j < nle; j += RPLAN_BLOCK) ahead[j] = 0;
+    for (int j = tid; j < RPLAN_WAVES * RPLAN_MAX_EXPERTS; j += RPLAN_BLOCK) (&in_wave[0][0])[j] = 0;
+    if (R < 0) R = rows();
+    lds_barrier();
+    if (first >= R) break;  // (uniform over the workgroup)
+    const bool ok = i < R;
+    const int le = floormod(mine, nle, magic);
+    for (int b = 0; b < first; b += SCAN_UNROLL * RPLAN_BLOCK) {
+      if (b > 0) {
+#pragma unroll
+        for (int u = 0; u < SCAN_UNROLL; ++u)
+          e2[u] = recv_meta[(size_t)min(b + tid + u * RPLAN_BLOCK, first - 1) * META];
+      }
+#pragma unroll
+      for (int u = 0; u < SCAN_UNROLL; ++u)
+        if (b + tid + u * RPLAN_BLOCK < first) atomicAdd(&ahead[floormod(e2[u], nle, magic)], 1);
+    }
+    int rank_in_wave = 0;
+    unsigned long long todo = __ballot(ok);
+    while (todo) {  // every lane of the wave runs the same number of rounds
+      const int head = __ffsll((long long)todo) - 1;
+      const int leader = __builtin_amdgcn_readlane(le, head);
+      const unsigned long long same = __ballot(ok && le == leader);
+      if (ok && le == leader) {
+        rank_in_wave = __popcll(same & lanes_below);
+        if (rank_in_wave == 0) in_wave[wave][leader] = __popcll(same);
+      }
+      todo &= ~same;
+    }
+    lds_barrier();
+    if (ok) {
+      int pos = ahead[le] + rank_in_wave;
+      for (int w = 0; w < wave; ++w) pos += in_wave[w][le];
+      row_pos[i] = pos;
+    }
+    lds_barrier();  // the tables are cleared again by the next tile
+  }
+}
+
+// POS: the position of every row inside its expert comes from `row_pos` (plan_recv_kernel);
+// the movers scan nothing.
+template <typename V, int NVW, bool PLAN, bool POS>
 __global__ __launch_bounds__(64 * ROWS) void dispatch_recv_kernel(
     const V* __restrict__ recv_buf, const int* __restrict__ recv_meta,
     const int* __restrict__ recv_counts, int W, int hint_rows, int capacity_rows, int nle,
     uint32_t magic, int max_recv, int row_vecs, int chunks, int* __restrict__ expert_num_tokens,
-    V* __restrict__ expert_x, int* __restrict__ expert_meta, int* __restrict__ plan) {
+    V* __restrict__ expert_x, int* __restrict__ expert_meta, int* __restrict__ plan,
+    const int* __restrict__ row_pos) {
   __shared__ int part[2 * ROWS * ROWS];
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const StridedKeys key{recv_meta, META};
@@ -868,6 +949,22 @@ __global__ __launch_bounds__(64 * ROWS) void dispatch_recv_kernel(
     const int i0 = grp * ROWS, i = i0 + wave;
     const int ic = min(i, limit - 1);
     const int base = c * (64 * NVW);
+
+    if constexpr (POS) {
+      const int e = recv_meta[(size_t)ic * META];
+      const int pos = row_pos[ic];
+      int m = 0;
+      if (c == 0 && lane < META) m = recv_meta[(size_t)ic * META + lane];
+      WavePayload<V, NVW> p;
+      p.load(recv_buf + (size_t)ic * row_vecs, base, row_vecs, lane);
+      const int R = rows_known();
+      if (i < R && (uint32_t)pos < (uint32_t)max_recv) {
+        const size_t row = (size_t)floormod(e, nle, magic) * max_recv + pos;
+        p.template store<(MOE_A2A_NT_RECV != 0)>(expert_x + row * row_vecs, base, row_vecs, lane);
+        if (c == 0 && lane < META) expert_meta[row * META + lane] = m;
+      }
+      return R;
+    }
 
     int re[ROWS];
 #pragma unroll
@@ -1295,11 +1392,37 @@ __device__ __forceinline__ void order_pair(int& ra, int& ka, int& rb, int& kb) {
   ra = r; ka = k;
 }
 
-template <typename V, int DT, int BLK, int NV>
+// Long streams: every workgroup of a token scanning the whole arriving stream makes the meta
+// reads grow with tokens x rows. return_map_kernel turns the stream into a table first: one
+// thread per arriving row writes its row number at entry_row[src_token * K + src_k]. A token's
+// workgroup then looks its K entries up instead of scanning (MAPPED below). An entry is taken
+// only if the meta row it points to names this token and this k NOW, so whatever an earlier
+// call left in the table can never be mistaken for an arrival; the table needs no clearing.
+// The one assumption is that no (token, k) pair arrives twice, which holds for every stream
+// the dispatch produced: with duplicates the table keeps one of them.
+__global__ __launch_bounds__(BLOCK) void return_map_kernel(
+    const int* __restrict__ recv_meta, const int* __restrict__ recv_counts, int W, int hint_rows,
+    int capacity_rows, int T, int K, int* __restrict__ entry_row) {
+  // the first row of a thread is loaded before the row count is known when it lies below the
+  // readable bound (the counts travel at the same time)
+  int i = blockIdx.x * BLOCK + threadIdx.x;
+  int tk[2] = {-1, -1};
+  bool loaded = i < hint_rows;
+  if (loaded) __builtin_memcpy(tk, recv_meta + (size_t)i * META + 2, 8);
+  const int R = min(sum_counts(recv_counts, W, capacity_rows), capacity_rows);
+  for (; i < R; i += gridDim.x * BLOCK) {
+    if (!loaded) __builtin_memcpy(tk, recv_meta + (size_t)i * META + 2, 8);
+    loaded = false;
+    if ((uint32_t)tk[0] < (uint32_t)T && (uint32_t)tk[1] < (uint32_t)K) entry_row[(size_t)tk[0] * K + tk[1]] = i;
+  }
+}
+
+template <typename V, int DT, int BLK, int NV, bool MAPPED>
 __global__ __launch_bounds__(BLK) void combine_recv_kernel(
     const V* __restrict__ recv_buf, const int* __restrict__ recv_meta,
     const int* __restrict__ recv_counts, int W, int hint_rows, int capacity_rows,
-    const float* __restrict__ weights, int T, int K, int row_vecs, int chunks, V* __restrict__ out, int accumulate) {
+    const float* __restrict__ weights, int T, int K, int row_vecs, int chunks, V* __restrict__ out, int accumulate,
+    const int* __restrict__ entry_row) {
   constexpr int N = Words<V>::N;
   constexpr int FAST = 8;  // addends ordered in registers
   __shared__ int hit_row[COMBINE_CAP], hit_k[COMBINE_CAP];
@@ -1362,7 +1485,23 @@ __global__ __launch_bounds__(BLK) void combine_recv_kernel(
 
     if (tid == 0) nhit = 0;
     lds_barrier();
-    if (R < 0) {
+    if constexpr (MAPPED) {
+      if (R < 0) R = min(lanes_hold_counts ? wave_sum(my_count) : sum_counts(recv_counts, W, capacity_rows), capacity_rows);
+      for (int k = tid; k < K; k += BLK) {
+        const int i = entry_row[(size_t)t * K + k];
+        if ((uint32_t)i < (uint32_t)R) {
+          int tk[2];
+          __builtin_memcpy(tk, recv_meta + (size_t)i * META + 2, 8);
+          if (tk[0] == t && tk[1] == k) {
+            const int p = atomicAdd(&nhit, 1);
+            if (p < COMBINE_CAP) {
+              hit_row[p] = i;
+              hit_k[p] = k;
+            }
+          }
+        }
+      }
+    } else if (R < 0) {
       // first item: one batch below the readable bound goes out before R is known
       const int spec = min(hint_rows, SCAN_UNROLL * BLK);
       scan(t, 0, spec);
@@ -1933,6 +2072,10 @@ int launch_status() { return hipGetLastError() == hipSuccess ? MOE_A2A_OK : MOE_
     }                                             \
   } while (0)
 
+#ifndef MOE_A2A_PLANNED_NVW
+#define MOE_A2A_PLANNED_NVW 4  // vectors per lane of a mover that scans nothing
+#endif
+
 // The send-back plan is kept by the lanes of one wave: one lane per source rank
 // in stage 2, one lane per local expert in stage 3.
 bool plan_supported(const moe_a2a_shape* s) {
@@ -1971,7 +2114,7 @@ long long group_items(long long rows, const Geometry& g) {
 
 extern "C" {
 
-const char* moe_a2a_version(void) { return "moe_a2a 0.4 gfx950"; }
+const char* moe_a2a_version(void) { return "moe_a2a 0.5 gfx950"; }
 
 #ifndef MOE_A2A_BUILD_ID
 #define MOE_A2A_BUILD_ID "unknown"
@@ -2084,10 +2227,16 @@ int moe_a2a_plan_send(const moe_a2a_shape* s, const int32_t* indices, int32_t nu
   return launch_status();
 }
 
-int moe_a2a_dispatch_recv(const moe_a2a_shape* s, const void* recv_buf, const int32_t* recv_meta,
-                          const int32_t* recv_counts, int32_t rows_hint, int32_t capacity_rows,
-                          int32_t* expert_num_tokens, void* expert_x, int32_t* expert_meta,
-                          int32_t* send_back_plan, void* stream) {
+}  // extern "C"
+
+namespace {
+
+// Stage 2; with `row_position` (capacity_rows ints of workspace) the positions come from a
+// planning launch and the movers scan nothing.
+int launch_dispatch_recv(const moe_a2a_shape* s, const void* recv_buf, const int32_t* recv_meta,
+                         const int32_t* recv_counts, int32_t rows_hint, int32_t capacity_rows,
+                         int32_t* expert_num_tokens, void* expert_x, int32_t* expert_meta,
+                         int32_t* send_back_plan, int32_t* row_position, void* stream) {
   if (!shape_ok(s) || rows_hint < 0 || capacity_rows < 0 || !recv_counts || !expert_num_tokens ||
       !expert_x || !expert_meta)
     return MOE_A2A_EINVAL;
@@ -2095,17 +2244,46 @@ int moe_a2a_dispatch_recv(const moe_a2a_shape* s, const void* recv_buf, const in
   if (rows_hint > capacity_rows) rows_hint = capacity_rows;
   if (capacity_rows > 0 && (!recv_buf || !recv_meta)) return MOE_A2A_EINVAL;
   if (!all_aligned(2, recv_buf, expert_x)) return MOE_A2A_EALIGN;
-  const Geometry g = geometry(s, recv_buf, expert_x);
+  Geometry g = geometry(s, recv_buf, expert_x);
+  hipStream_t st = (hipStream_t)stream;
+  const bool planned = send_back_plan && plan_supported(s);
+  if (row_position && g.nle <= RPLAN_MAX_EXPERTS && capacity_rows > 0) {
+    // no scan to repeat per chunk: a row is split among more waves, as in the planned stage 3
+    if (g.vec16 && g.nvw > MOE_A2A_PLANNED_NVW) {
+      g.nvw = MOE_A2A_PLANNED_NVW;
+      g.wchunks = (g.row_vecs + 64 * g.nvw - 1) / (64 * g.nvw);
+    }
+    if (!items_fit((long long)g.nle * g.max_recv, g.wchunks)) return MOE_A2A_EINVAL;
+    const int tiles = (int)std::min<long long>(((long long)rows_hint + RPLAN_BLOCK - 1) / RPLAN_BLOCK + 1, 1 << 16);
+    plan_recv_kernel<<<tiles, RPLAN_BLOCK, 0, st>>>(recv_meta, recv_counts, s->world_size, rows_hint,
+                                                    capacity_rows, g.nle, g.magic, row_position);
+    const int grid = g.nle + mover_blocks(group_items(rows_hint, g));
+#define LAUNCH_P(V, NVW, PLAN)                                                              \
+  dispatch_recv_kernel<V, NVW, PLAN, true><<<grid, 64 * ROWS, 0, st>>>(                     \
+      (const V*)recv_buf, recv_meta, recv_counts, s->world_size, rows_hint, capacity_rows,   \
+      g.nle, g.magic, g.max_recv, g.row_vecs, g.wchunks, expert_num_tokens, (V*)expert_x,    \
+      expert_meta, send_back_plan, row_position)
+#define LAUNCH(V, NVW)                     \
+  do {                                     \
+    if (planned) LAUNCH_P(V, NVW, true);   \
+    else LAUNCH_P(V, NVW, false);          \
+  } while (0)
+    if (!g.vec16) LAUNCH(uint16_t, 16);
+    else if (g.nvw == 1) LAUNCH(b128, 1);
+    else if (g.nvw == 2) LAUNCH(b128, 2);
+    else LAUNCH(b128, 4);
+#undef LAUNCH
+#undef LAUNCH_P
+    return launch_status();
+  }
   // the stream can hold at most nle * max_recv rows that fit the expert buffers
   if (!items_fit((long long)g.nle * g.max_recv, g.wchunks)) return MOE_A2A_EINVAL;
   const int grid = g.nle + mover_blocks(group_items(rows_hint, g));
-  hipStream_t st = (hipStream_t)stream;
-  const bool planned = send_back_plan && plan_supported(s);
 #define LAUNCH_P(V, NVW, PLAN)                                                              \
-  dispatch_recv_kernel<V, NVW, PLAN><<<grid, 64 * ROWS, 0, st>>>(                           \
+  dispatch_recv_kernel<V, NVW, PLAN, false><<<grid, 64 * ROWS, 0, st>>>(                    \
       (const V*)recv_buf, recv_meta, recv_counts, s->world_size, rows_hint, capacity_rows,   \
       g.nle, g.magic, g.max_recv, g.row_vecs, g.wchunks, expert_num_tokens, (V*)expert_x,    \
-      expert_meta, send_back_plan)
+      expert_meta, send_back_plan, nullptr)
 #define LAUNCH(V, NVW)                     \
   do {                                     \
     if (planned) LAUNCH_P(V, NVW, true);   \
@@ -2115,6 +2293,27 @@ int moe_a2a_dispatch_recv(const moe_a2a_shape* s, const void* recv_buf, const in
 #undef LAUNCH
 #undef LAUNCH_P
   return launch_status();
+}
+
+}  // namespace
+
+extern "C" {
+
+int moe_a2a_dispatch_recv(const moe_a2a_shape* s, const void* recv_buf, const int32_t* recv_meta,
+                          const int32_t* recv_counts, int32_t rows_hint, int32_t capacity_rows,
+                          int32_t* expert_num_tokens, void* expert_x, int32_t* expert_meta,
+                          int32_t* send_back_plan, void* stream) {
+  return launch_dispatch_recv(s, recv_buf, recv_meta, recv_counts, rows_hint, capacity_rows,
+                              expert_num_tokens, expert_x, expert_meta, send_back_plan, nullptr, stream);
+}
+
+int moe_a2a_dispatch_recv_long(const moe_a2a_shape* s, const void* recv_buf, const int32_t* recv_meta,
+                               const int32_t* recv_counts, int32_t rows_hint, int32_t capacity_rows,
+                               int32_t* expert_num_tokens, void* expert_x, int32_t* expert_meta,
+                               int32_t* send_back_plan, int32_t* row_position, void* stream) {
+  if (!row_position) return MOE_A2A_EINVAL;
+  return launch_dispatch_recv(s, recv_buf, recv_meta, recv_counts, rows_hint, capacity_rows,
+                              expert_num_tokens, expert_x, expert_meta, send_back_plan, row_position, stream);
 }
 
 int moe_a2a_dispatch_recv_static(const moe_a2a_shape* s, const void* recv_buf,
@@ -2150,9 +2349,6 @@ int moe_a2a_combine_send(const moe_a2a_shape* s, const void* expert_y, const int
   // The planned path has no scan to repeat per chunk, so a row can be split among more waves:
   // 4 vectors per lane (a 256-vector chunk per wave) made the whole step 0.5 us shorter at
   // H = 7168 than the 14 the scan path uses; 2, 6 and 8 were no better than 14.
-#ifndef MOE_A2A_PLANNED_NVW
-#define MOE_A2A_PLANNED_NVW 4
-#endif
   if (planned && g.vec16 && g.nvw > MOE_A2A_PLANNED_NVW) {
     g.nvw = MOE_A2A_PLANNED_NVW;
     g.wchunks = (g.row_vecs + 64 * g.nvw - 1) / (64 * g.nvw);
@@ -2177,10 +2373,16 @@ int moe_a2a_combine_send(const moe_a2a_shape* s, const void* expert_y, const int
   return launch_status();
 }
 
-int moe_a2a_combine_recv(const moe_a2a_shape* s, const void* recv_buf, const int32_t* recv_meta,
-                         const int32_t* recv_counts, int32_t rows_hint, int32_t capacity_rows,
-                         const float* weights, int32_t num_tokens, void* out_tokens,
-                         int32_t accumulate, int32_t dtype, void* stream) {
+}  // extern "C"
+
+namespace {
+
+// Stage 4; with `entry_row` (num_tokens * K ints of workspace) a launch of its own first maps
+// every (token, k) to its arriving row and the workgroups look their rows up instead of scanning.
+int launch_combine_recv(const moe_a2a_shape* s, const void* recv_buf, const int32_t* recv_meta,
+                        const int32_t* recv_counts, int32_t rows_hint, int32_t capacity_rows,
+                        const float* weights, int32_t num_tokens, void* out_tokens,
+                        int32_t accumulate, int32_t dtype, int32_t* entry_row, void* stream) {
   if (!shape_ok(s) || num_tokens < 0 || num_tokens > s->max_num_tokens || !recv_counts ||
       rows_hint < 0 || capacity_rows < 0)
     return MOE_A2A_EINVAL;
@@ -2205,10 +2407,23 @@ int moe_a2a_combine_recv(const moe_a2a_shape* s, const void* recv_buf, const int
   const int grid = mover_blocks((long long)num_tokens * chunks);
   hipStream_t st = (hipStream_t)stream;
   const int K = s->experts_per_token, W = s->world_size;
+  const bool mapped = entry_row != nullptr && capacity_rows > 0;
+  if (mapped) {
+    const int mgrid = (int)std::min<long long>(((long long)rows_hint + BLOCK - 1) / BLOCK + 1, 1 << 16);
+    return_map_kernel<<<mgrid, BLOCK, 0, st>>>(recv_meta, recv_counts, W, rows_hint, capacity_rows,
+                                               num_tokens, K, entry_row);
+  }
 #define LAUNCH(V, DT, BLK, NV)                                                               \
-  combine_recv_kernel<V, DT, BLK, NV><<<grid, BLK, 0, st>>>(                                 \
-      (const V*)recv_buf, recv_meta, recv_counts, W, rows_hint, capacity_rows, weights,      \
-      num_tokens, K, g.row_vecs, chunks, (V*)out_tokens, accumulate)
+  do {                                                                                       \
+    if (mapped)                                                                              \
+      combine_recv_kernel<V, DT, BLK, NV, true><<<grid, BLK, 0, st>>>(                       \
+          (const V*)recv_buf, recv_meta, recv_counts, W, rows_hint, capacity_rows, weights,  \
+          num_tokens, K, g.row_vecs, chunks, (V*)out_tokens, accumulate, entry_row);         \
+    else                                                                                     \
+      combine_recv_kernel<V, DT, BLK, NV, false><<<grid, BLK, 0, st>>>(                      \
+          (const V*)recv_buf, recv_meta, recv_counts, W, rows_hint, capacity_rows, weights,  \
+          num_tokens, K, g.row_vecs, chunks, (V*)out_tokens, accumulate, nullptr);           \
+  } while (0)
 #define PICK_SHAPE(V, DT)                       \
   do {                                          \
     if (nv == 1) { LAUNCH(V, DT, BLOCK, 1); }   \
@@ -2224,6 +2439,27 @@ int moe_a2a_combine_recv(const moe_a2a_shape* s, const void* recv_buf, const int
 #undef PICK_SHAPE
 #undef LAUNCH
   return launch_status();
+}
+
+}  // namespace
+
+extern "C" {
+
+int moe_a2a_combine_recv(const moe_a2a_shape* s, const void* recv_buf, const int32_t* recv_meta,
+                         const int32_t* recv_counts, int32_t rows_hint, int32_t capacity_rows,
+                         const float* weights, int32_t num_tokens, void* out_tokens,
+                         int32_t accumulate, int32_t dtype, void* stream) {
+  return launch_combine_recv(s, recv_buf, recv_meta, recv_counts, rows_hint, capacity_rows, weights,
+                             num_tokens, out_tokens, accumulate, dtype, nullptr, stream);
+}
+
+int moe_a2a_combine_recv_long(const moe_a2a_shape* s, const void* recv_buf, const int32_t* recv_meta,
+                              const int32_t* recv_counts, int32_t rows_hint, int32_t capacity_rows,
+                              const float* weights, int32_t num_tokens, void* out_tokens,
+                              int32_t accumulate, int32_t dtype, int32_t* entry_row, void* stream) {
+  if (!entry_row) return MOE_A2A_EINVAL;
+  return launch_combine_recv(s, recv_buf, recv_meta, recv_counts, rows_hint, capacity_rows, weights,
+                             num_tokens, out_tokens, accumulate, dtype, entry_row, stream);
 }
 
 int moe_a2a_expert_scale(const moe_a2a_shape* s, const void* expert_x,

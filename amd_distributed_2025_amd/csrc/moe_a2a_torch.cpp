@@ -103,7 +103,8 @@ void a2a_plan_send(std::vector<int64_t> shape, torch::Tensor indices, int64_t nu
 void a2a_dispatch_recv(std::vector<int64_t> shape, torch::Tensor recv_buf, torch::Tensor recv_meta,
                        torch::Tensor recv_counts, int64_t rows_hint, torch::Tensor expert_num_tokens,
                        torch::Tensor expert_x, torch::Tensor expert_meta,
-                       c10::optional<torch::Tensor> send_back_plan, int64_t stream) {
+                       c10::optional<torch::Tensor> send_back_plan,
+                       c10::optional<torch::Tensor> row_position, int64_t stream) {
   const moe_a2a_shape s = shape_of(shape);
   const auto dt = rows_type(recv_buf, "recv_buf");
   const int64_t nle = s.world_size > 0 ? s.num_experts / s.world_size : 0;
@@ -119,6 +120,15 @@ void a2a_dispatch_recv(std::vector<int64_t> shape, torch::Tensor recv_buf, torch
   need(expert_meta, "expert_meta", torch::kInt32, padded * MOE_A2A_META_DIM, &recv_buf);
   if (send_back_plan.has_value())
     need(*send_back_plan, "send_back_plan", torch::kInt32, 2 * (int64_t)s.num_experts, &recv_buf);
+  if (row_position.has_value()) {  // long streams: positions from a planning launch
+    need(*row_position, "row_position", torch::kInt32, capacity, &recv_buf);
+    status(moe_a2a_dispatch_recv_long(&s, recv_buf.data_ptr(), ints(recv_meta), ints(recv_counts),
+                                      to_i32(rows_hint, "rows_hint"), to_i32(capacity, "capacity_rows"),
+                                      ints(expert_num_tokens), expert_x.data_ptr(), ints(expert_meta),
+                                      ints_or_null(send_back_plan), ints(*row_position), stream_of(stream)),
+           "moe_a2a_dispatch_recv_long");
+    return;
+  }
   status(moe_a2a_dispatch_recv(&s, recv_buf.data_ptr(), ints(recv_meta), ints(recv_counts),
                                to_i32(rows_hint, "rows_hint"), to_i32(capacity, "capacity_rows"),
                                ints(expert_num_tokens), expert_x.data_ptr(), ints(expert_meta),
@@ -153,7 +163,8 @@ void a2a_combine_send(std::vector<int64_t> shape, torch::Tensor expert_y, torch:
 
 void a2a_combine_recv(std::vector<int64_t> shape, torch::Tensor recv_buf, torch::Tensor recv_meta,
                       torch::Tensor recv_counts, int64_t rows_hint, torch::Tensor weights, int64_t num_tokens,
-                      torch::Tensor out_tokens, bool accumulate, int64_t stream) {
+                      torch::Tensor out_tokens, bool accumulate, c10::optional<torch::Tensor> entry_row,
+                      int64_t stream) {
   const moe_a2a_shape s = shape_of(shape);
   const auto dt = rows_type(out_tokens, "out_tokens");
   need(out_tokens, "out_tokens", dt, num_tokens * s.hidden_dim);
@@ -163,6 +174,16 @@ void a2a_combine_recv(std::vector<int64_t> shape, torch::Tensor recv_buf, torch:
                                     recv_meta.numel() / MOE_A2A_META_DIM);
   need(recv_counts, "recv_counts", torch::kInt32, s.world_size, &out_tokens);
   need(weights, "weights", torch::kFloat32, num_tokens * s.experts_per_token, &out_tokens);
+  if (entry_row.has_value()) {  // long streams: rows looked up in a (token, k) -> row table
+    need(*entry_row, "entry_row", torch::kInt32, num_tokens * s.experts_per_token, &out_tokens);
+    status(moe_a2a_combine_recv_long(&s, recv_buf.data_ptr(), ints(recv_meta), ints(recv_counts),
+                                     to_i32(std::min(rows_hint, capacity), "rows_hint"),
+                                     to_i32(capacity, "capacity_rows"), weights.data_ptr<float>(),
+                                     to_i32(num_tokens, "num_tokens"), out_tokens.data_ptr(), accumulate ? 1 : 0,
+                                     dtype_code(dt), ints(*entry_row), stream_of(stream)),
+           "moe_a2a_combine_recv_long");
+    return;
+  }
   status(moe_a2a_combine_recv(&s, recv_buf.data_ptr(), ints(recv_meta), ints(recv_counts),
                               to_i32(std::min(rows_hint, capacity), "rows_hint"), to_i32(capacity, "capacity_rows"),
                               weights.data_ptr<float>(), to_i32(num_tokens, "num_tokens"), out_tokens.data_ptr(),

@@ -180,6 +180,17 @@ WORKLOADS = {
 }
 
 
+# The C4 shape with two, four and six times the tokens per rank (4096 to 12288 rows sent per rank):
+# not part of the task's lists; bench.py times them to show how the path scales with the row count.
+LARGE_WORKLOADS = {
+    "C4x2": dict(WORKLOADS["C4"], max_num_tokens=512),
+    "C4x4": dict(WORKLOADS["C4"], max_num_tokens=1024),
+    "C4x6": dict(WORKLOADS["C4"], max_num_tokens=1536),
+    # 32768 rows per rank: two ranks with C4's 32 local experts each and 4096 tokens
+    "W2x16": dict(WORKLOADS["C4"], world_size=2, num_experts=64, max_num_tokens=4096),
+}
+
+
 def generate_world(workload: dict, seed: int, device=None):
     """Inputs of every rank of one job: list of `input_t`, one per rank."""
     spec = dict(workload)

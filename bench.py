@@ -56,7 +56,7 @@ def parse_args():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", default="C4", choices=["C1", "C2", "C3", "C4", "C5"])
+    ap.add_argument("--workload", default="C4", choices=["C1", "C2", "C3", "C4", "C5", "C4x2", "C4x4", "C4x6", "W2x16"])
     ap.add_argument("--seed", type=int, default=2025)
     ap.add_argument("--rank", type=int, default=0, help="rank whose share of the job is the timed step")
     ap.add_argument("--mode", default="graph", choices=["graph", "eager"],
@@ -69,6 +69,9 @@ def parse_args():
     ap.add_argument("--no-rank-sweep", action="store_true", help="time only --rank, not every rank of the job")
     ap.add_argument("--no-placement-plan", action="store_true",
                     help="combine_send ranks its rows by scanning instead of using dispatch_recv's plan")
+    ap.add_argument("--long-stream-rows", type=int, default=None,
+                    help="row count above which the receive halves take the long-stream entry points "
+                         "(default: the host class's own threshold)")
     ap.add_argument("--alone", action="store_true",
                     help="also time every kernel back to back with itself (warm inputs)")
     return ap.parse_args()
@@ -120,7 +123,8 @@ def main():
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
 
-    wl = WORKLOADS[args.workload]
+    from amd_distributed_2025_amd.task import LARGE_WORKLOADS
+    wl = {**WORKLOADS, **LARGE_WORKLOADS}[args.workload]
     world = generate_world(wl, args.seed)
     cfg = world[0][0]
     W, K, H = len(world), cfg.experts_per_token, cfg.hidden_dim
@@ -130,7 +134,8 @@ def main():
         sys.exit(2)
 
     # ---- set-up: the whole job once, so every rank's inbound buffers hold the peers' segments
-    lw = LocalWorld(cfg, W, device=dev, reuse_placement=not args.no_placement_plan)
+    lw = LocalWorld(cfg, W, device=dev, reuse_placement=not args.no_placement_plan,
+                    long_stream_rows=args.long_stream_rows)
     ys0 = [y.clone() for y in lw.run(data)]
     torch.cuda.synchronize()
 

@@ -202,9 +202,11 @@ def test_torch_extension_wraps_every_entry_point():
     assert m.a2a_version() == _lib.load().moe_a2a_version().decode()
     wrapped = {"moe_" + f for f in EXT_FUNCTIONS}
     # not wrapped: the message lookup, and the variant for callers that cannot allocate (it hands
-    # back a raw device address, which has no torch::Tensor form)
+    # back a raw device address, which has no torch::Tensor form); the long-stream variants are
+    # what a2a_dispatch_recv / a2a_combine_recv call when they are handed the table argument
     assert wrapped == set(declared_functions()) - {"moe_a2a_strerror", "moe_a2a_build_id",
-                                                   "moe_a2a_dispatch_recv_static"}
+                                                   "moe_a2a_dispatch_recv_static",
+                                                   "moe_a2a_dispatch_recv_long", "moe_a2a_combine_recv_long"}
     source = (ROOT / "amd_distributed_2025_amd" / "csrc" / "moe_a2a_torch.cpp").read_text()
     for f in EXT_FUNCTIONS:
         assert hasattr(m, f), f

@@ -1,0 +1,159 @@
+"""The long-stream entry points (moe_a2a_dispatch_recv_long, moe_a2a_combine_recv_long): positions
+from a planning launch instead of a scan in every workgroup. They must give what the one-launch
+entry points give and what the oracle says, bit for bit, at every size; `long_stream_rows=0`
+sends every receive half through them, however short its stream."""
+import numpy as np
+import pytest
+import torch
+
+from amd_distributed_2025_amd import LocalWorld, WORKLOADS, generate_world
+from amd_distributed_2025_amd.all2all import LONG_STREAM_ROWS
+from tests.helpers import bits, run_oracle
+from tests.test_gpu_parity import DEV, EDGE, assert_rank_matches, to_dev
+
+pytestmark = pytest.mark.gpu
+
+
+def run_long(world, long_stream_rows=0, exact_hints=True, accumulate=False, reuse_placement=True,
+             binding="ctypes", lw=None):
+    cfg = world[0][0]
+    if lw is None:
+        lw = LocalWorld(cfg, len(world), device=DEV, exact_hints=exact_hints, reuse_placement=reuse_placement,
+                        binding=binding, long_stream_rows=long_stream_rows)
+    ys = lw.run([d for _, d, _, _ in to_dev(world)], accumulate=accumulate)
+    torch.cuda.synchronize()
+    tr = run_oracle(world)
+    for r in range(len(world)):
+        T = world[r][1].num_tokens
+        assert_rank_matches(lw.trace[r], tr[r], T, cfg.experts_per_token, f"rank {r}")
+        assert np.array_equal(bits(ys[r]), tr[r].y)
+    return lw
+
+
+@pytest.mark.parametrize("name", ["C1", "C2", "C3", "C4", "C5"])
+def test_workloads_through_the_long_stream_entry_points(name):
+    print(f"long-stream workload {name}", flush=True)
+    run_long(generate_world(WORKLOADS[name], 2025))
+
+
+@pytest.mark.parametrize("name", sorted(EDGE))
+def test_edge_shapes_through_the_long_stream_entry_points(name):
+    print(f"long-stream edge {name}", flush=True)
+    spec = dict(routing="uniform", weights="rand")
+    spec.update(EDGE[name])
+    run_long(generate_world(spec, 77))
+
+
+def test_extension_binding_and_loose_hints():
+    world = generate_world(WORKLOADS["C3"], 5)
+    run_long(world, binding="ext")
+    run_long(world, exact_hints=False, accumulate=True, reuse_placement=False)
+
+
+def test_streams_above_the_threshold_take_them_by_default():
+    """16384 rows sent and about as many received per rank, many planning tiles, skewed
+    routing; nothing forced: the host class picks the long-stream entry points from the row
+    count."""
+    spec = dict(world_size=4, num_experts=64, experts_per_token=8, hidden_dim=264, max_num_tokens=2048,
+                num_tokens="full", routing="zipf", weights="softmax", dtype="bf16")
+    world = generate_world(spec, 4)
+    assert spec["max_num_tokens"] * spec["experts_per_token"] > max(LONG_STREAM_ROWS.values())
+    lw = run_long(world, long_stream_rows=None)
+    assert any("row_position" in a._ws for a in lw.ranks)  # (skewed routing: not every rank receives that many)
+    assert all("entry_row" in a._ws for a in lw.ranks)
+    # and the one-launch entry points agree on the same job
+    short = LocalWorld(world[0][0], 4, device=DEV, long_stream_rows=1 << 30)
+    ys = short.run([d for _, d, _, _ in to_dev(world)])
+    torch.cuda.synchronize()
+    assert not any("row_position" in a._ws or "entry_row" in a._ws for a in short.ranks)
+    for r in range(4):
+        assert torch.equal(ys[r], lw.trace[r]["y"][: world[r][1].num_tokens])
+
+
+def test_tables_left_by_an_earlier_job_do_no_harm():
+    """The (token, k) -> row table and the position table are never cleared. A second, smaller
+    job on the same objects finds the first job's entries in them and must not use any."""
+    spec = dict(world_size=4, num_experts=16, experts_per_token=4, hidden_dim=264, max_num_tokens=96,
+                num_tokens="full", routing="uniform", weights="rand", dtype="fp16")
+    lw = run_long(generate_world(spec, 1))
+    small = dict(spec, num_tokens="uniform")
+    for seed in (2, 3):
+        run_long(generate_world(small, seed), lw=lw)
+
+
+def test_random_small_jobs_through_the_long_stream_entry_points():
+    rng = np.random.default_rng(777)
+    for case in range(24):
+        W = int(rng.choice([1, 2, 3, 4, 8, 16]))
+        nle = int(rng.choice([1, 2, 5, 32, 65, 130, 300]))  # (300: beyond the planner's tables, scans instead)
+        E = W * nle
+        K = int(rng.integers(1, min(E, 9) + 1))
+        H = int(rng.choice([8, 24, 100, 256, 520, 1032, 4104]))
+        max_T = int(rng.integers(1, 300))
+        spec = dict(world_size=W, num_experts=E, experts_per_token=K, hidden_dim=H, max_num_tokens=max_T,
+                    num_tokens=str(rng.choice(["uniform", "full", "reference"])),
+                    routing=str(rng.choice(["uniform", "zipf"])),
+                    weights=str(rng.choice(["rand", "softmax"])),
+                    dtype=str(rng.choice(["bf16", "fp16"])))
+        print(f"long-stream random job {case}: {spec}", flush=True)
+        run_long(generate_world(spec, 500 + case), exact_hints=bool(case % 2))
+
+
+def test_overflowing_expert_drops_the_same_rows():
+    """Every entry routed to expert 0: positions reach past max_recv and those rows are not
+    stored, exactly as with the scanning movers."""
+    spec = dict(world_size=2, num_experts=4, experts_per_token=4, hidden_dim=64, max_num_tokens=6,
+                num_tokens="full", routing="uniform", weights="rand", dtype="bf16")
+    world = generate_world(spec, 11)
+    cfg = world[0][0]
+    outs = []
+    for long_rows in (0, 1 << 30):
+        lw = LocalWorld(cfg, len(world), device=DEV, long_stream_rows=long_rows)
+        data = [d.to(DEV) for _, d, _, _ in world]
+        for d in data:
+            d.indices = torch.zeros_like(d.indices)
+        ys = lw.run(data)
+        torch.cuda.synchronize()
+        tr = lw.trace[0]
+        assert int(tr["expert_num_tokens"][0]) > lw.ranks[0].max_recv
+        n = int(tr["back_counts"].sum())
+        outs.append([tr["expert_num_tokens"].cpu().numpy(), tr["back_counts"].cpu().numpy(),
+                     tr["back_meta"][:n].cpu().numpy(), bits(tr["back_buf"][:n])] + [bits(y) for y in ys])
+    for a, b in zip(*outs):
+        assert np.array_equal(a, b)
+
+
+def test_graph_replays_of_the_long_stream_step():
+    world = generate_world(WORKLOADS["C3"], 12)
+    cfg = world[0][0]
+    dev = [d.to(DEV) for _, d, _, _ in world]
+    lw = LocalWorld(cfg, 8, device=DEV, long_stream_rows=0)
+    eager = [y.clone() for y in lw.run(dev)]
+    a, d0, g = lw.ranks[0], dev[0], lw.trace[0]
+    R = int(g["recv_counts"].sum().item())
+    y = a._buf("y", (cfg.max_num_tokens, cfg.hidden_dim), cfg.out_dtype)
+
+    def step():
+        a.dispatch_send(d0.x, d0.indices)
+        a.dispatch_recv(g["recv_counts"], g["recv_buf"], g["recv_meta"], R)
+        a.expert_scale(g["expert_x"], g["expert_num_tokens"], R)
+        a.combine_send(g["expert_meta"], g["expert_y"], g["expert_num_tokens"], R)
+        a.combine_recv(y, d0.weights, g["ret_counts"], g["ret_buf"], g["ret_meta"], accumulate=False)
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        step()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        step()
+    for i in range(3):
+        y.fill_(float(i))
+        a._ws["entry_row"].fill_(i)      # whatever the tables hold before a replay
+        a._ws["row_position"].fill_(-1)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(y[: d0.num_tokens], eager[0]), f"replay {i}"
