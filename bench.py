@@ -18,7 +18,8 @@ mean over exactly `--steps` graph replays between two synchronisations; `step_us
 are taken over batches of the same replays timed with events. `hot_path_us` is the time of the four path
 launches by themselves: HIP events on the launch stream around a graph that holds `--kernel-reps` times
 dispatch_send, dispatch_recv, combine_send, combine_recv and nothing else, every input resident where
-the step leaves it. The cost of one of them is that time minus the time of the same graph without it;
+the step leaves it; `hot_path_launch_floor_us` is the same graph on a job without rows (what four
+launches cost when they move nothing). The cost of one of them is that time minus the time of the same graph without it;
 `roofline` prices the slowest against HBM peak with the algorithmic bytes of its stage.
 `hot_path_us_in_step` is the whole step minus a step of the three stand-ins alone. `ranks` repeats the
 hot-path figure for every rank of the job (their received row counts differ); `cpu_baseline` is the
@@ -253,6 +254,28 @@ def main():
 
     hot_us, kern, total_alg = path_costs(stages, T, R, alone=args.alone)
     reps = args.kernel_reps
+
+    # What a launch of this path costs with nothing to move: the same four entry points in the same
+    # kind of graph on a job without rows (no tokens sent, zero counts everywhere). It is the part of
+    # a small workload's time that no kernel change can win back.
+    def launch_floor():
+        a, g = lw.ranks[r0], lw.trace[r0]
+        zc = torch.zeros(W, dtype=torch.int32, device=dev)
+        zn = torch.zeros(a.num_local_experts, dtype=torch.int32, device=dev)
+        d0 = data[r0]
+        fns = [
+            lambda: a.dispatch_send(d0.x[:0], d0.indices[:0]),
+            lambda: a.dispatch_recv(zc, g["recv_buf"], g["recv_meta"], 0),
+            lambda: a.combine_send(g["expert_meta"], g["expert_y"], zn, 0),
+            lambda: a.combine_recv(y, d0.weights[:1], zc, g["ret_buf"], g["ret_meta"], accumulate=True),
+        ]
+        us = time_graph(graph_of(fns, reps), reps)
+        for _, fn in stages:  # put every buffer back as a full step leaves it
+            fn()
+        torch.cuda.synchronize()
+        return us
+
+    floor_us = launch_floor()
     full_us = time_graph(graph_of([fn for _, fn in stages], reps), reps)
     standins_us = time_graph(graph_of([fn for n, fn in stages if n not in PATH], reps), reps)
     dominant = max(PATH, key=lambda n: kern[n]["us"])
@@ -284,6 +307,8 @@ def main():
         "hot_path_us": round(hot_us, 3),
         "hot_path_measure": f"graph of {reps} x the four path launches, HIP events, median of 9",
         "hot_path_us_in_step": round(full_us - standins_us, 3),
+        "hot_path_launch_floor_us": round(floor_us, 3),
+        "hot_path_launch_floor_measure": "the same graph of the four entry points on a job without rows",
         "hot_path_kernel_sum_us": round(sum(kern[n]["us"] for n in PATH), 3),
         "hot_path_alg_bytes": total_alg,
         "hot_path_gbps": round(total_alg / hot_us * 1e-3, 1),
