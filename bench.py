@@ -28,7 +28,8 @@ host cores, with the vectorised numpy statement beside it; `custom_kernel_wall_u
 reference's entry point (which steps all ranks of the job on this one GPU). `expert_gemm` is the
 grouped GEMM a model would run between the two halves, on this rank's expert-major rows and random
 weights: one launch between HIP events, priced against HBM peak (it streams every weight once) with
-its matrix rate beside it.
+its matrix rate beside it. `linear` is the per-rank product of the reference's gemm-rs task at the
+largest shape of its benchmark list, priced against the dense bf16 matrix rate.
 """
 from __future__ import annotations
 
@@ -66,7 +67,10 @@ def parse_args():
                     help="repetitions of the launches inside each timing graph")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="target CPU time of the cpu_baseline sample")
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
-    ap.add_argument("--no-gemm", action="store_true", help="skip the grouped GEMM row")
+    ap.add_argument("--no-gemm", action="store_true", help="skip the grouped GEMM and linear rows")
+    ap.add_argument("--no-floor", action="store_true",
+                    help="skip the launch-floor measurement (its launches without rows would count into a "
+                         "profiler's per-kernel averages)")
     ap.add_argument("--no-rank-sweep", action="store_true", help="time only --rank, not every rank of the job")
     ap.add_argument("--no-placement-plan", action="store_true",
                     help="combine_send ranks its rows by scanning instead of using dispatch_recv's plan")
@@ -275,7 +279,7 @@ def main():
         torch.cuda.synchronize()
         return us
 
-    floor_us = launch_floor()
+    floor_us = None if args.no_floor else launch_floor()
     full_us = time_graph(graph_of([fn for _, fn in stages], reps), reps)
     standins_us = time_graph(graph_of([fn for n, fn in stages if n not in PATH], reps), reps)
     dominant = max(PATH, key=lambda n: kern[n]["us"])
@@ -307,7 +311,7 @@ def main():
         "hot_path_us": round(hot_us, 3),
         "hot_path_measure": f"graph of {reps} x the four path launches, HIP events, median of 9",
         "hot_path_us_in_step": round(full_us - standins_us, 3),
-        "hot_path_launch_floor_us": round(floor_us, 3),
+        "hot_path_launch_floor_us": None if floor_us is None else round(floor_us, 3),
         "hot_path_launch_floor_measure": "the same graph of the four entry points on a job without rows",
         "hot_path_kernel_sum_us": round(sum(kern[n]["us"] for n in PATH), 3),
         "hot_path_alg_bytes": total_alg,
@@ -396,6 +400,47 @@ def main():
             "measure": "HIP events around single launches, median of 10",
         }
         del wts
+
+    # ---- the gemm-rs task's per-rank product (gemm-rs/reference.py:54-57) at the largest shape of
+    # its benchmark list (m = n = 8192, k = 29568 over 8 ranks, no bias): matrix-core bound
+    if not args.no_gemm:
+        from amd_distributed_2025_amd import gemm_rs
+
+        m, n, k_job = 8192, 8192, 29568
+        lin = gemm_rs.generate_input(0, 8, m, n, k_job, False, 42, device=dev)
+        lin_out = torch.empty(m, n, dtype=torch.bfloat16, device=dev)
+        ev = [torch.cuda.Event(enable_timing=True) for _ in range(2)]
+
+        def timed(fn, n_runs=10):
+            ts = []
+            for i in range(n_runs + 3):
+                ev[0].record()
+                fn()
+                ev[1].record()
+                ev[1].synchronize()
+                if i >= 3:
+                    ts.append(ev[0].elapsed_time(ev[1]) * 1e3)
+            return statistics.median(ts)
+
+        lin_us = timed(lambda: gemm_rs.local_product(lin, out=lin_out))
+        torch_us = timed(lambda: torch.matmul(lin[0], lin[1].T))
+        k_loc = k_job // 8
+        flop = 2 * m * n * k_loc
+        rows = torch.arange(0, m, 257, device=dev)
+        want = lin[0][rows].float() @ lin[1].float().T
+        got = lin_out[rows].float()
+        out["linear"] = {
+            "shape": {"m": m, "n": n, "k_per_rank": k_loc, "bias": False},
+            "us": round(lin_us, 1), "flop": flop,
+            "roofline": {"bound": "mfma", "achieved": round(flop / lin_us * 1e-6, 1), "peak": MFMA_PEAK_TFLOPS,
+                         "unit": "TFLOP/s", "frac": round(flop / lin_us * 1e-6 / MFMA_PEAK_TFLOPS, 4)},
+            "torch_matmul_us": round(torch_us, 1),
+            "torch_matmul_tflops": round(flop / torch_us * 1e-6, 1),
+            "max_rel_err_vs_fp32_matmul": float(((got - want).abs() / (want.abs() + 1e-3)).max().item()),
+            "measure": "HIP events around single launches, median of 10; torch.matmul (the vendor "
+                       "library, what the reference calls) timed the same way beside it",
+        }
+        del lin, lin_out
 
     # ---- CPU baseline: the row-by-row torch statement of the same step on the host cores
     if not args.no_cpu:
