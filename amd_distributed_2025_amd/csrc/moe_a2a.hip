@@ -1746,23 +1746,29 @@ template <> struct Mfma32x32x16<MOE_A2A_F16> {
 #ifndef MOE_A2A_GEMM_OCC
 #define MOE_A2A_GEMM_OCC 3
 #endif
+#ifndef MOE_A2A_GEMM_OCC4
+#define MOE_A2A_GEMM_OCC4 2  // workgroups per compute unit with blocks of 128 tokens
+#endif
 #ifndef MOE_A2A_GEMM_DEPTH
 #define MOE_A2A_GEMM_DEPTH 2
 #endif
 constexpr int BUFFER_RAW_32BIT = 0x00020000;  // word 3 of a gfx9 buffer descriptor: raw buffer of 32-bit data
 constexpr int GEMM_COLS = 128;   // output columns per workgroup, 32 per wave
 constexpr int GEMM_KSTEP = 64;   // input elements per step: 8 vectors of 16 bytes per row
+#ifndef MOE_A2A_GEMM_DEPTH4
+#define MOE_A2A_GEMM_DEPTH4 3  // with blocks of 128 tokens (two workgroups per unit: 655 against 675 us at C4)
+#endif
 constexpr int GEMM_DEPTH = MOE_A2A_GEMM_DEPTH;  // steps between a load and its use
 
 // x [groups, max_rows, K], w [groups, N, K], bias [groups, N] or null, y [groups, max_rows, N];
 // rows_of_group null: every group has max_rows rows (a plain dense product when groups == 1).
 template <int DT, int TJ>
-__global__ __launch_bounds__(BLOCK, TJ <= 2 ? MOE_A2A_GEMM_OCC : 2) void expert_gemm_kernel(
+__global__ __launch_bounds__(BLOCK, TJ <= 2 ? MOE_A2A_GEMM_OCC : MOE_A2A_GEMM_OCC4) void expert_gemm_kernel(
     const b128* __restrict__ expert_x, const int* __restrict__ expert_num_tokens,
     const b128* __restrict__ weights, const uint16_t* __restrict__ bias, uint16_t* __restrict__ expert_y,
     int nle, int max_recv, int N, int K, int col_tiles) {
   constexpr int TOK = TJ * 32;               // tokens per block
-  constexpr int D = GEMM_DEPTH;
+  constexpr int D = TJ >= 4 ? MOE_A2A_GEMM_DEPTH4 : GEMM_DEPTH;
   __shared__ b128 xs[D][TOK * 8];            // D steps of TOK tokens x 8 vectors
   __shared__ b128 ws[NWAVES][32 * 8];        // per wave: one step of its 32 weight rows x 8 vectors
   __shared__ int red[NWAVES];
@@ -1944,6 +1950,129 @@ __global__ __launch_bounds__(BLOCK, TJ <= 2 ? MOE_A2A_GEMM_OCC : 2) void expert_
             __builtin_memcpy(out + g * 8, two, 8);
           }
         }
+      }
+    }
+  }
+}
+
+// ---------------------------------------------------------------- product with few rows
+//
+// Y[M, N] = X[M, K] @ W[N, K]^T with so few rows that tiles of 128 columns do not fill the chip
+// (M = 64, N = 7168: 56 workgroups). Here a workgroup owns only 32 output columns x one block of
+// tokens, and its four waves split K: wave w takes steps w, w + 4, ... of 64 elements, streams
+// its own slices of the 32 weight rows and of the token rows (both 8 lanes per 128-byte line,
+// turned into MFMA layout through LDS private to the wave: no barrier in the loop), and keeps
+// partial sums in registers. At the end the partial sums meet in LDS and are added in a fixed
+// order (wave 0 + 1 + 2 + 3), so results do not depend on scheduling.
+
+template <int DT, int TJ>
+__global__ __launch_bounds__(BLOCK, TJ <= 2 ? 3 : 2) void skinny_gemm_kernel(
+    const b128* __restrict__ X, const b128* __restrict__ Wt, const uint16_t* __restrict__ bias,
+    uint16_t* __restrict__ Y, int M, int N, int K, int col_units) {
+  constexpr int TOK = TJ * 32;
+  constexpr int XL = TJ * 4;  // token loads per lane and step: TOK rows x 8 vectors over 64 lanes
+  __shared__ b128 wsl[NWAVES][32 * 8];
+  __shared__ b128 xsl[NWAVES][TOK * 8];
+  const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
+  const int row_vecs = K / 8, row_bytes = K * 2, steps = (K + GEMM_KSTEP - 1) / GEMM_KSTEP;
+  const int tail_vecs = row_vecs - (steps - 1) * 8;
+  const int rb = blockIdx.x / col_units, cu = blockIdx.x - rb * col_units;
+  const int t0 = rb * TOK, n0 = cu * 32, live = M - t0;
+
+  const __amdgpu_buffer_rsrc_t wbuf = __builtin_amdgcn_make_buffer_rsrc(
+      (void*)(Wt + (size_t)n0 * row_vecs), 0, 32 * row_bytes, BUFFER_RAW_32BIT);
+  const __amdgpu_buffer_rsrc_t xbuf = __builtin_amdgcn_make_buffer_rsrc(
+      (void*)(X + (size_t)t0 * row_vecs), 0, min(live, TOK) * row_bytes, BUFFER_RAW_32BIT);
+  constexpr int OUT_OF_RANGE = 0x40000000;
+  // load i of a lane: row sub + 8 * i, the vector that belongs in physical slot `slot` of that row
+  const int sub = lane >> 3, slot = lane & 7;
+  auto vec_of = [&](int row) { return slot ^ ((row >> 1) & 7); };
+  const int r = lane & 31, kb = lane >> 5, read_swz = (r >> 1) & 7;
+
+  f32x16 acc[TJ] = {};
+  b128 wv[2][4], xv[2][XL];
+  auto load = [&](int set, int step) {
+    const int at = min(step, steps - 1);  // past the end: the last step again, unused
+    const bool last = at == steps - 1;
+    const int soff = at * (GEMM_KSTEP * 2);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int row = sub + 8 * i, vec = vec_of(row);
+      wv[set][i] = __builtin_amdgcn_raw_buffer_load_b128(
+          wbuf, row * row_bytes + vec * 16 + (last && vec >= tail_vecs ? OUT_OF_RANGE : 0), soff, 0);
+    }
+#pragma unroll
+    for (int i = 0; i < XL; ++i) {
+      const int row = sub + 8 * i, vec = vec_of(row);
+      xv[set][i] = __builtin_amdgcn_raw_buffer_load_b128(
+          xbuf, row * row_bytes + vec * 16 + (last && vec >= tail_vecs ? OUT_OF_RANGE : 0), soff, 0);
+    }
+  };
+  auto compute = [&](int set) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) wsl[wave][(sub + 8 * i) * 8 + slot] = wv[set][i];
+#pragma unroll
+    for (int i = 0; i < XL; ++i) xsl[wave][(sub + 8 * i) * 8 + slot] = xv[set][i];
+    b128 a[4];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) a[q] = wsl[wave][r * 8 + ((kb * 4 + q) ^ read_swz)];
+#pragma unroll
+    for (int q = 0; q < 4; ++q)
+#pragma unroll
+      for (int j = 0; j < TJ; ++j) {
+        if (j * 32 < live) {
+          const b128 tok = xsl[wave][(j * 32 + r) * 8 + ((kb * 4 + q) ^ read_swz)];
+          acc[j] = Mfma32x32x16<DT>::mma(a[q], tok, acc[j]);
+        }
+      }
+  };
+
+  load(0, wave);
+  load(1, wave + NWAVES);
+  for (int s = wave; s < steps; s += 2 * NWAVES) {
+    compute(0);
+    load(0, s + 2 * NWAVES);
+    if (s + NWAVES < steps) compute(1);
+    load(1, s + 3 * NWAVES);
+  }
+
+  // partial sums to LDS (a wave's region holds exactly its TJ x 16 floats per lane), then wave j
+  // adds up token tile j in the order of the waves and writes it out
+  float* mine = reinterpret_cast<float*>(xsl[wave]);
+#pragma unroll
+  for (int j = 0; j < TJ; ++j)
+#pragma unroll
+    for (int e = 0; e < 16; ++e) mine[(j * 16 + e) * 64 + lane] = acc[j][e];
+  __syncthreads();
+  if (wave < TJ && wave * 32 < live) {
+    const int j = wave;
+    float c[16];
+#pragma unroll
+    for (int e = 0; e < 16; ++e) {
+      float sum = reinterpret_cast<const float*>(xsl[0])[(j * 16 + e) * 64 + lane];
+#pragma unroll
+      for (int w = 1; w < NWAVES; ++w)
+        sum = __fadd_rn(sum, reinterpret_cast<const float*>(xsl[w])[(j * 16 + e) * 64 + lane]);
+      c[e] = sum;
+    }
+    // this lane: token r of tile j, output columns n0 + g*8 + kb*4 + 0..3, g < 4
+    const int token = t0 + j * 32 + r;
+    if (token < M) {
+      uint16_t* out = Y + (size_t)token * N + n0 + kb * 4;
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        uint32_t two[2] = {Pair16<DT>::canonical(Pair16<DT>::round(c[g * 4 + 0], c[g * 4 + 1])),
+                           Pair16<DT>::canonical(Pair16<DT>::round(c[g * 4 + 2], c[g * 4 + 3]))};
+        if (bias) {
+          uint32_t b2[2];
+          __builtin_memcpy(b2, bias + n0 + kb * 4 + g * 8, 8);
+#pragma unroll
+          for (int h = 0; h < 2; ++h)
+            two[h] = Pair16<DT>::canonical(Pair16<DT>::round(
+                __fadd_rn(Pair16<DT>::lo(two[h]), Pair16<DT>::lo(b2[h])),
+                __fadd_rn(Pair16<DT>::hi(two[h]), Pair16<DT>::hi(b2[h]))));
+        }
+        __builtin_memcpy(out + g * 8, two, 8);
       }
     }
   }
@@ -2830,6 +2959,39 @@ int launch_dense_gemm(const void* a, const void* b, const void* bias, void* c, i
   return launch_status();
 }
 
+#ifndef MOE_A2A_SKINNY_MAX_TILES
+#define MOE_A2A_SKINNY_MAX_TILES 192  // tiles of 128 columns below which K is split inside the workgroup
+#endif
+
+// Products whose tiles of 128 columns would leave compute units idle: 32 columns per workgroup,
+// K split over its waves. MOE_A2A_NOT_DENSE when the grouped kernel is the better fit.
+int launch_skinny_gemm(const void* x, const void* w, const void* bias, void* y, int M, int N, int K,
+                       int dtype, hipStream_t st) {
+  if (dtype != MOE_A2A_F16 && dtype != MOE_A2A_BF16) return MOE_A2A_EINVAL;
+  if (N % 32 != 0 || K % 8 != 0) return MOE_A2A_EINVAL;
+  if (!all_aligned(16, x, w, y) || !all_aligned(8, bias)) return MOE_A2A_EALIGN;
+  if ((long long)K * 2 * 128 >= (1 << 30)) return MOE_A2A_NOT_DENSE;
+  const int tj = M > 64 ? 4 : 2;
+  const long long row_blocks = ((long long)M + tj * 32 - 1) / (tj * 32);
+  const long long wide_tiles = row_blocks * ((N + GEMM_COLS - 1) / GEMM_COLS);
+  const int steps = (K + GEMM_KSTEP - 1) / GEMM_KSTEP;
+  if (wide_tiles >= MOE_A2A_SKINNY_MAX_TILES || steps < 2 * NWAVES) return MOE_A2A_NOT_DENSE;
+  const long long grid = row_blocks * (N / 32);
+  if (grid > INT_MAX / 2) return MOE_A2A_NOT_DENSE;
+#define LAUNCH_K(DT, TJ)                                                                           \
+  skinny_gemm_kernel<DT, TJ><<<(int)grid, BLOCK, 0, st>>>((const b128*)x, (const b128*)w,         \
+                                                          (const uint16_t*)bias, (uint16_t*)y, M, N, K, N / 32)
+  if (dtype == MOE_A2A_BF16) {
+    if (tj == 2) LAUNCH_K(MOE_A2A_BF16, 2);
+    else LAUNCH_K(MOE_A2A_BF16, 4);
+  } else {
+    if (tj == 2) LAUNCH_K(MOE_A2A_F16, 2);
+    else LAUNCH_K(MOE_A2A_F16, 4);
+  }
+#undef LAUNCH_K
+  return launch_status();
+}
+
 }  // namespace
 
 extern "C" {
@@ -2851,6 +3013,8 @@ int moe_a2a_linear(const void* input, const void* weight, const void* bias, int3
   if (m == 0) return MOE_A2A_OK;
   const int dense = launch_dense_gemm(input, weight, bias, output, m, n, k, dtype, (hipStream_t)stream);
   if (dense != MOE_A2A_NOT_DENSE) return dense;
+  const int skinny = launch_skinny_gemm(input, weight, bias, output, m, n, k, dtype, (hipStream_t)stream);
+  if (skinny != MOE_A2A_NOT_DENSE) return skinny;
   return launch_grouped_gemm(input, nullptr, weight, bias, output, 1, m, m, n, k, dtype,
                              (hipStream_t)stream);
 }

@@ -63,7 +63,9 @@ def test_task_shapes(m, n, k, has_bias, seed):
 
 
 @pytest.mark.parametrize("dt", [torch.bfloat16, torch.float16], ids=["bf16", "fp16"])
-@pytest.mark.parametrize("m,n,k", [(1, 32, 8), (70, 96, 72), (129, 160, 360), (300, 2880, 200), (64, 64, 64)])
+# (the last four: few rows and many steps of K, where a workgroup's waves split K among them)
+@pytest.mark.parametrize("m,n,k", [(1, 32, 8), (70, 96, 72), (129, 160, 360), (300, 2880, 200), (64, 64, 64),
+                                   (1, 32, 512), (64, 96, 520), (70, 64, 1000), (200, 160, 1096)])
 def test_small_integers_with_bias_are_exact(m, n, k, dt):
     print(f"linear integers m={m} n={n} k={k} {dt}", flush=True)
     rng = np.random.default_rng(m * n + k)
@@ -79,7 +81,8 @@ def test_small_integers_with_bias_are_exact(m, n, k, dt):
     out = torch.full((m + 2, n), 777.0, dtype=dt, device=DEV)
     gemm_rs.local_product((pad[1:m + 1], wpad[1:n + 1], bias), out=out[1:m + 1])
     torch.cuda.synchronize()
-    want = x @ w.T + b[None, :]  # |values| <= 360 + 8: integers both 16-bit types hold
+    want = x @ w.T + b[None, :]
+    assert np.abs(want).max() <= 256 and np.abs(x @ w.T).max() <= 256  # integers both 16-bit types hold
     assert np.array_equal(out[1:m + 1].float().cpu().numpy(), want.astype(np.float32))
     assert (out[0] == 777.0).all() and (out[m + 1] == 777.0).all()
     no_bias = gemm_rs.local_product((pad[1:m + 1], wpad[1:n + 1], None))
