@@ -2944,12 +2944,22 @@ int launch_dense_gemm(const void* a, const void* b, const void* bias, void* c, i
   if ((long long)K * 2 * 256 >= (1 << 30)) return MOE_A2A_NOT_DENSE;  // 32-bit byte offsets inside a tile's rows
   constexpr size_t lds_bytes = 2 * (BM + BN) * 8 * sizeof(b128);
   const int grid = (int)(tiles_m * tiles_n);
+  // the tile buffers are more LDS than a kernel gets by default: allowed once per GPU and kernel
+  int gpu = -1;
+  if (hipGetDevice(&gpu) != hipSuccess || gpu < 0 || gpu >= MAX_GPUS) return MOE_A2A_ELAUNCH;
 #define LAUNCH_D(DT)                                                                              \
   do {                                                                                            \
     auto kernel = dense_gemm_kernel<DT, 2, 2, 4, 4>;                                              \
-    static const hipError_t allowed =                                                             \
-        hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes); \
-    if (allowed != hipSuccess) return MOE_A2A_ELAUNCH;                                            \
+    static bool allowed[MAX_GPUS] = {};                                                           \
+    {                                                                                             \
+      std::lock_guard<std::mutex> lock(static_plan_mutex);                                        \
+      if (!allowed[gpu]) {                                                                        \
+        if (hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize,  \
+                                (int)lds_bytes) != hipSuccess)                                    \
+          return MOE_A2A_ELAUNCH;                                                                 \
+        allowed[gpu] = true;                                                                      \
+      }                                                                                           \
+    }                                                                                             \
     kernel<<<grid, 256, lds_bytes, st>>>((const b128*)a, (const b128*)b, (const uint16_t*)bias,   \
                                          (uint16_t*)c, M, N, K, (int)tiles_m, (int)tiles_n);      \
   } while (0)
