@@ -1868,14 +1868,18 @@ __global__ __launch_bounds__(BLOCK, TJ <= 2 ? MOE_A2A_GEMM_OCC : MOE_A2A_GEMM_OC
     auto load_x = [&](int set, int step) {
       const int at = min(step, steps - 1);
       const bool last = at == steps - 1;
+      // (load i holds tokens 32 * i .. 32 * i + 31 of the block: a tile of 32 tokens without a valid
+      // token is neither loaded nor parked nor multiplied)
 #pragma unroll
       for (int i = 0; i < TJ; ++i)
-        xv[set][i] = __builtin_amdgcn_raw_buffer_load_b128(xbuf, xoff[i] + (last ? xpast : 0),
-                                                           at * (GEMM_KSTEP * 2), 0);
+        if (i * 32 < live)
+          xv[set][i] = __builtin_amdgcn_raw_buffer_load_b128(xbuf, xoff[i] + (last ? xpast : 0),
+                                                             at * (GEMM_KSTEP * 2), 0);
     };
     auto park_x = [&](int set) {
 #pragma unroll
-      for (int i = 0; i < TJ; ++i) xs[set][tid + BLOCK * i] = xv[set][i];
+      for (int i = 0; i < TJ; ++i)
+        if (i * 32 < live) xs[set][tid + BLOCK * i] = xv[set][i];
     };
     auto compute = [&](int set) {
 #pragma unroll

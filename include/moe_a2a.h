@@ -342,11 +342,17 @@ int moe_a2a_expert_gemm(const moe_a2a_shape* shape, const void* expert_x,
  * output[m, n] = input[m, k] @ weight[n, k]^T (+ bias[n]): the product one rank
  * computes in the reference's gemm-rs task before the reduce-scatter
  * (gemm-rs/reference.py:54-57: `torch.matmul(input, weight.T)`, then
- * `output + bias`). Same kernel as moe_a2a_expert_gemm with one group of m rows.
- * All tensors are of the 16-bit type `dtype` (MOE_A2A_F16 / MOE_A2A_BF16), row-major,
- * k contiguous in input and weight. Accumulation is float32 with one rounding
- * to the 16-bit type; a bias is then added to that rounded value and the sum
- * rounded again, which is what the two torch statements do. bias may be NULL.
+ * `output + bias`). All tensors are of the 16-bit type `dtype` (MOE_A2A_F16 /
+ * MOE_A2A_BF16), row-major, k contiguous in input and weight. Accumulation is
+ * float32 with one rounding to the 16-bit type; a bias is then added to that
+ * rounded value and the sum rounded again, which is what the two torch
+ * statements do. bias may be NULL.
+ * One of three kernels runs, picked from the shape alone (so a shape always
+ * gives the same bits): from 128 output tiles of 256 x 256 on, a kernel bound
+ * by the matrix cores (four waves of 128 x 128 per tile); with so few rows that
+ * tiles of 128 columns would number fewer than 192, a kernel whose workgroups
+ * own 32 columns and split k over their waves (partial sums added in a fixed
+ * order); otherwise the kernel of moe_a2a_expert_gemm with one group of m rows.
  * Limits: n a multiple of 32, k a multiple of 8, input / weight / output 16-byte
  * and bias 8-byte aligned (MOE_A2A_EINVAL / EALIGN). m == 0 is a no-op.
  * The reduce-scatter that follows in the reference (gemm-rs/reference.py:58-59)
