@@ -51,10 +51,10 @@ def test_extension_binding_and_loose_hints():
 
 
 def test_streams_above_the_threshold_take_them_by_default():
-    """16384 rows sent and about as many received per rank, many planning tiles, skewed
+    """20480 rows sent and about as many received per rank, many planning tiles, skewed
     routing; nothing forced: the host class picks the long-stream entry points from the row
     count."""
-    spec = dict(world_size=4, num_experts=64, experts_per_token=8, hidden_dim=264, max_num_tokens=2048,
+    spec = dict(world_size=4, num_experts=64, experts_per_token=8, hidden_dim=264, max_num_tokens=2560,
                 num_tokens="full", routing="zipf", weights="softmax", dtype="bf16")
     world = generate_world(spec, 4)
     assert spec["max_num_tokens"] * spec["experts_per_token"] > max(LONG_STREAM_ROWS.values())
@@ -68,6 +68,22 @@ def test_streams_above_the_threshold_take_them_by_default():
     assert not any("row_position" in a._ws or "entry_row" in a._ws for a in short.ranks)
     for r in range(4):
         assert torch.equal(ys[r], lw.trace[r]["y"][: world[r][1].num_tokens])
+
+
+def test_repeated_expert_ids_and_many_ranks():
+    """Entries of a token that name the same expert keep their k order, also through the
+    long-stream entry points; a job of 16 ranks."""
+    spec = dict(world_size=16, num_experts=32, experts_per_token=6, hidden_dim=136, max_num_tokens=200,
+                num_tokens="full", routing="uniform", weights="rand", dtype="bf16")
+    world = generate_world(spec, 99)
+    rng = np.random.default_rng(5)
+    for _, d, r, _ in world:
+        ids = rng.integers(0, 32, tuple(d.indices.shape)).astype(np.int32)
+        ids[r] = 7
+        ids[r + 4, :3] = 31
+        d.indices = torch.from_numpy(ids)
+    run_long(world)
+    run_long(world, reuse_placement=False, exact_hints=False)
 
 
 def test_tables_left_by_an_earlier_job_do_no_harm():

@@ -597,8 +597,9 @@ def test_repeated_expert_ids_inside_a_token():
         run_and_compare(world, reuse_placement=plan)
 
 
+@pytest.mark.parametrize("long_rows", [None, 0], ids=["one_launch", "long_stream"])
 @pytest.mark.parametrize("K", [2, 6])
-def test_expert_ids_outside_the_range_are_set_aside(K):
+def test_expert_ids_outside_the_range_are_set_aside(K, long_rows):
     """Ids below 0 or at/above E name no destination. Their rows must land behind all
     destinations' rows without disturbing them, and the result must equal the oracle's on a job
     where those entries point at a real expert with weight 0 (an addend of +0 changes nothing)."""
@@ -621,7 +622,7 @@ def test_expert_ids_outside_the_range_are_set_aside(K):
         ds.x = d.x
     want = run_oracle(substitute)
     cfg = world[0][0]
-    lw = LocalWorld(cfg, W, device=DEV)
+    lw = LocalWorld(cfg, W, device=DEV, long_stream_rows=long_rows)
     ys = lw.run([d.to(DEV) for _, d, _, _ in world])
     torch.cuda.synchronize()
     nle = E // W
