@@ -65,7 +65,10 @@ def test_task_shapes(m, n, k, has_bias, seed):
 @pytest.mark.parametrize("dt", [torch.bfloat16, torch.float16], ids=["bf16", "fp16"])
 # (the last four: few rows and many steps of K, where a workgroup's waves split K among them)
 @pytest.mark.parametrize("m,n,k", [(1, 32, 8), (70, 96, 72), (129, 160, 360), (300, 2880, 200), (64, 64, 64),
-                                   (1, 32, 512), (64, 96, 520), (70, 64, 1000), (200, 160, 1096)])
+                                   (1, 32, 512), (64, 96, 520), (70, 64, 1000), (200, 160, 1096),
+                                   # many rows: tiles of 256 x 256 with ragged last tiles in both directions,
+                                   # one and several steps of K, a K tail
+                                   (3000, 2944, 72), (2050, 4128, 200), (4100, 2080, 8)])
 def test_small_integers_with_bias_are_exact(m, n, k, dt):
     print(f"linear integers m={m} n={n} k={k} {dt}", flush=True)
     rng = np.random.default_rng(m * n + k)
