@@ -35,9 +35,10 @@ META_DIM = 5
 # Streams of more rows than this take the entry points that rank in a planning launch of their
 # own (moe_a2a_dispatch_recv_long, moe_a2a_combine_recv_long); shorter ones the one-launch
 # entry points, whose movers rank by scanning. Results are the same; the second launch costs
-# about 5 us, which both halves have earned back at 4096 rows (measured at hidden_dim 7168: equal
-# there, 7 % ahead at 8192 rows, 17 % at 12288, 40 % at 32768).
-LONG_STREAM_ROWS = {"dispatch": 4096, "combine": 4096}
+# about 5 us, which the combine has earned back at 4096 rows and the dispatch, whose scans hide
+# behind its payload for longer, at 8192 (measured at hidden_dim 7168; at 12288 rows the two
+# together are 17 % ahead, at 32768 rows 40 %).
+LONG_STREAM_ROWS = {"dispatch": 8192, "combine": 4096}
 
 
 def _stream(device) -> int:
