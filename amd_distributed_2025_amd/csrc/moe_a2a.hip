@@ -1761,16 +1761,22 @@ constexpr int GEMM_DEPTH = MOE_A2A_GEMM_DEPTH;  // steps between a load and its 
 
 // x [groups, max_rows, K], w [groups, N, K], bias [groups, N] or null, y [groups, max_rows, N];
 // rows_of_group null: every group has max_rows rows (a plain dense product when groups == 1).
-template <int DT, int TJ>
-__global__ __launch_bounds__(BLOCK, TJ <= 2 ? MOE_A2A_GEMM_OCC : MOE_A2A_GEMM_OCC4) void expert_gemm_kernel(
+// GW waves per workgroup, 32 output columns each: every workgroup of an expert pulls the expert's
+// token rows through its own L1, so wider workgroups halve that traffic (GW = 8: one workgroup of
+// 512 lanes per compute unit instead of two of 256).
+template <int DT, int TJ, int GW>
+__global__ __launch_bounds__(64 * GW, GW == 8 ? 1 : TJ <= 2 ? MOE_A2A_GEMM_OCC : MOE_A2A_GEMM_OCC4) void expert_gemm_kernel(
     const b128* __restrict__ expert_x, const int* __restrict__ expert_num_tokens,
     const b128* __restrict__ weights, const uint16_t* __restrict__ bias, uint16_t* __restrict__ expert_y,
     int nle, int max_recv, int N, int K, int col_tiles) {
   constexpr int TOK = TJ * 32;               // tokens per block
   constexpr int D = TJ >= 4 ? MOE_A2A_GEMM_DEPTH4 : GEMM_DEPTH;
   __shared__ b128 xs[D][TOK * 8];            // D steps of TOK tokens x 8 vectors
-  __shared__ b128 ws[NWAVES][32 * 8];        // per wave: one step of its 32 weight rows x 8 vectors
-  __shared__ int red[NWAVES];
+  constexpr int THREADS = 64 * GW;
+  constexpr int XL = TOK * 8 / THREADS;       // token loads of a lane per step (64 * GW / 8 rows each)
+  static_assert(XL >= 1 && XL * THREADS == TOK * 8, "whole loads");
+  __shared__ b128 ws[GW][32 * 8];            // per wave: one step of its 32 weight rows x 8 vectors
+  __shared__ int red[GW];
   __shared__ int home[2];
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const int row_vecs = K / 8, steps = (K + GEMM_KSTEP - 1) / GEMM_KSTEP;
@@ -1780,7 +1786,7 @@ __global__ __launch_bounds__(BLOCK, TJ <= 2 ? MOE_A2A_GEMM_OCC : MOE_A2A_GEMM_OC
   // Blocks of tokens per expert, summed over the run of experts this thread owns and scanned over
   // the workgroup: block number g of the launch belongs to the thread with begin <= g < begin + mine.
   auto blocks_of = [=](int le) { return (rows_of(le) + TOK - 1) / TOK; };
-  const int per = (nle + BLOCK - 1) / BLOCK;
+  const int per = (nle + THREADS - 1) / THREADS;
   const int run_b = min(tid * per, nle), run_e = min(run_b + per, nle);
   int mine = 0;
   for (int le = run_b; le < run_e; ++le) mine += blocks_of(le);
@@ -1791,7 +1797,7 @@ __global__ __launch_bounds__(BLOCK, TJ <= 2 ? MOE_A2A_GEMM_OCC : MOE_A2A_GEMM_OC
     lds_barrier();
     int off = 0, total = 0;
 #pragma unroll
-    for (int w = 0; w < NWAVES; ++w) {
+    for (int w = 0; w < GW; ++w) {
       off += w < wave ? red[w] : 0;
       total += red[w];
     }
@@ -1823,7 +1829,7 @@ __global__ __launch_bounds__(BLOCK, TJ <= 2 ? MOE_A2A_GEMM_OCC : MOE_A2A_GEMM_OC
     const int le = __builtin_amdgcn_readfirstlane(home[0]);
     const int rows = __builtin_amdgcn_readfirstlane(rows_of(le));
     const int t0 = (rb - __builtin_amdgcn_readfirstlane(home[1])) * TOK;  // first token of the block (t0 < rows)
-    const int n0 = ct * GEMM_COLS + __builtin_amdgcn_readfirstlane(wave) * 32;  // first output column of this wave
+    const int n0 = ct * (GW * 32) + __builtin_amdgcn_readfirstlane(wave) * 32;  // first output column of this wave
     const bool cols_valid = n0 < N;                      // the last tile of columns may be partly empty
     const int nw = min(n0, N - 32);                      // (a wave without columns reads valid memory)
 
@@ -1841,7 +1847,7 @@ __global__ __launch_bounds__(BLOCK, TJ <= 2 ? MOE_A2A_GEMM_OCC : MOE_A2A_GEMM_OC
     const __amdgpu_buffer_rsrc_t xbuf = __builtin_amdgcn_make_buffer_rsrc(
         (void*)(expert_x + ((size_t)le * max_recv + t0) * row_vecs), 0, min(live, TOK) * row_bytes, BUFFER_RAW_32BIT);
     constexpr int OUT_OF_RANGE = 0x40000000;
-    int woff[4], wslot[4], xoff[TJ], wpast[2];
+    int woff[4], wslot[4], xoff[XL], wpast[2];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const int row = sub + 8 * i, vec = slot ^ ((row >> 1) & 7);
@@ -1849,13 +1855,14 @@ __global__ __launch_bounds__(BLOCK, TJ <= 2 ? MOE_A2A_GEMM_OCC : MOE_A2A_GEMM_OC
       wslot[i] = row * 8 + slot;
       if (i < 2) wpast[i] = vec >= tail_vecs ? OUT_OF_RANGE : 0;  // (loads i and i + 2 take the same vector)
     }
-    const int xrow = tid >> 3, xvec = slot ^ ((xrow >> 1) & 7);  // (32*i does not change bits 1..3)
+    constexpr int XROWS = THREADS / 8;  // token rows one load of the workgroup covers: 32 or 64
+    const int xrow = tid >> 3, xvec = slot ^ ((xrow >> 1) & 7);  // (XROWS * i does not change bits 1..3)
     const int xpast = xvec >= tail_vecs ? OUT_OF_RANGE : 0;
 #pragma unroll
-    for (int i = 0; i < TJ; ++i) xoff[i] = (xrow + 32 * i) * row_bytes + xvec * 16;
+    for (int i = 0; i < XL; ++i) xoff[i] = (xrow + XROWS * i) * row_bytes + xvec * 16;
 
     f32x16 acc[TJ] = {};
-    b128 wv[D][4], xv[D][TJ];
+    b128 wv[D][4], xv[D][XL];
     auto load_w = [&](int set, int step) {
       const int at = min(step, steps - 1);  // past the end: the last step again, unused
       const bool last = at == steps - 1;
@@ -1867,18 +1874,18 @@ __global__ __launch_bounds__(BLOCK, TJ <= 2 ? MOE_A2A_GEMM_OCC : MOE_A2A_GEMM_OC
     auto load_x = [&](int set, int step) {
       const int at = min(step, steps - 1);
       const bool last = at == steps - 1;
-      // (load i holds tokens 32 * i .. 32 * i + 31 of the block: a tile of 32 tokens without a valid
-      // token is neither loaded nor parked nor multiplied)
+      // (load i holds tokens XROWS * i .. of the block: a load without a valid token is neither
+      // issued nor parked, and a tile of 32 tokens without one is not multiplied)
 #pragma unroll
-      for (int i = 0; i < TJ; ++i)
-        if (i * 32 < live)
+      for (int i = 0; i < XL; ++i)
+        if (i * XROWS < live)
           xv[set][i] = __builtin_amdgcn_raw_buffer_load_b128(xbuf, xoff[i] + (last ? xpast : 0),
                                                              at * (GEMM_KSTEP * 2), 0);
     };
     auto park_x = [&](int set) {
 #pragma unroll
-      for (int i = 0; i < TJ; ++i)
-        if (i * 32 < live) xs[set][tid + BLOCK * i] = xv[set][i];
+      for (int i = 0; i < XL; ++i)
+        if (i * XROWS < live) xs[set][tid + THREADS * i] = xv[set][i];
     };
     auto compute = [&](int set) {
 #pragma unroll
@@ -2910,22 +2917,31 @@ int launch_grouped_gemm(const void* x, const int32_t* rows_of_group, const void*
   if (!all_aligned(16, x, w, y) || !all_aligned(8, bias)) return MOE_A2A_EALIGN;
   // per-lane byte offsets inside a block of tokens and inside a wave's 32 weight rows are 32-bit
   if ((long long)K * 2 * 128 >= (1 << 30) || max_rows > INT_MAX / 2) return MOE_A2A_EINVAL;
-  const int col_tiles = (N + GEMM_COLS - 1) / GEMM_COLS;
   const int tj = rows_hint > (long long)MOE_A2A_GEMM_ROWS_FOR_128 * groups ? 4 : 2;
   // every group can end in a partly filled block of tokens; the kernel strides over what the hint misses
   const long long row_blocks = rows_hint / (tj * 32) + groups;
+  // Workgroups of 256 columns (8 waves) pull an expert's token rows through half as many L1s as
+  // workgroups of 128; taken when blocks hold 128 tokens and there are still tiles for every unit.
+#ifndef MOE_A2A_GEMM_WIDE_MIN_TILES
+#define MOE_A2A_GEMM_WIDE_MIN_TILES 512
+#endif
+  const bool wide = tj == 4 && row_blocks * ((N + 255) / 256) >= MOE_A2A_GEMM_WIDE_MIN_TILES;
+  const int cols = wide ? 256 : GEMM_COLS;
+  const int col_tiles = (N + cols - 1) / cols;
   if ((max_rows / 64 + 1) * groups * col_tiles > INT_MAX / 2) return MOE_A2A_EINVAL;
   const int grid = mover_blocks(row_blocks * col_tiles);
-#define LAUNCH_G(DT, TJ)                                                                          \
-  expert_gemm_kernel<DT, TJ><<<grid, BLOCK, 0, st>>>((const b128*)x, rows_of_group, (const b128*)w, \
-                                                     (const uint16_t*)bias, (uint16_t*)y, groups,  \
-                                                     (int)max_rows, N, K, col_tiles)
+#define LAUNCH_G(DT, TJ, GW)                                                                          \
+  expert_gemm_kernel<DT, TJ, GW><<<grid, 64 * GW, 0, st>>>((const b128*)x, rows_of_group, (const b128*)w, \
+                                                           (const uint16_t*)bias, (uint16_t*)y, groups,  \
+                                                           (int)max_rows, N, K, col_tiles)
   if (dtype == MOE_A2A_BF16) {
-    if (tj == 2) LAUNCH_G(MOE_A2A_BF16, 2);
-    else LAUNCH_G(MOE_A2A_BF16, 4);
+    if (tj == 2) LAUNCH_G(MOE_A2A_BF16, 2, 4);
+    else if (wide) LAUNCH_G(MOE_A2A_BF16, 4, 8);
+    else LAUNCH_G(MOE_A2A_BF16, 4, 4);
   } else {
-    if (tj == 2) LAUNCH_G(MOE_A2A_F16, 2);
-    else LAUNCH_G(MOE_A2A_F16, 4);
+    if (tj == 2) LAUNCH_G(MOE_A2A_F16, 2, 4);
+    else if (wide) LAUNCH_G(MOE_A2A_F16, 4, 8);
+    else LAUNCH_G(MOE_A2A_F16, 4, 4);
   }
 #undef LAUNCH_G
   return launch_status();
