@@ -25,6 +25,7 @@
 #include <stdint.h>
 #include <limits.h>
 #include <algorithm>
+#include <cmath>
 #include <mutex>
 #include <type_traits>
 
@@ -1765,7 +1766,7 @@ constexpr int GEMM_DEPTH = MOE_A2A_GEMM_DEPTH;  // steps between a load and its 
 // token rows through its own L1, so wider workgroups halve that traffic (GW = 8: one workgroup of
 // 512 lanes per compute unit instead of two of 256).
 template <int DT, int TJ, int GW>
-__global__ __launch_bounds__(64 * GW, GW == 8 ? 1 : TJ <= 2 ? MOE_A2A_GEMM_OCC : MOE_A2A_GEMM_OCC4) void expert_gemm_kernel(
+__global__ __launch_bounds__(64 * GW, GW > 4 ? 1 : TJ <= 2 ? MOE_A2A_GEMM_OCC : MOE_A2A_GEMM_OCC4) void expert_gemm_kernel(
     const b128* __restrict__ expert_x, const int* __restrict__ expert_num_tokens,
     const b128* __restrict__ weights, const uint16_t* __restrict__ bias, uint16_t* __restrict__ expert_y,
     int nle, int max_recv, int N, int K, int col_tiles) {
@@ -1773,8 +1774,11 @@ __global__ __launch_bounds__(64 * GW, GW == 8 ? 1 : TJ <= 2 ? MOE_A2A_GEMM_OCC :
   constexpr int D = TJ >= 4 ? MOE_A2A_GEMM_DEPTH4 : GEMM_DEPTH;
   __shared__ b128 xs[D][TOK * 8];            // D steps of TOK tokens x 8 vectors
   constexpr int THREADS = 64 * GW;
-  constexpr int XL = TOK * 8 / THREADS;       // token loads of a lane per step (64 * GW / 8 rows each)
-  static_assert(XL >= 1 && XL * THREADS == TOK * 8, "whole loads");
+  // the token rows of a step are fetched and parked by all lanes when their number divides the
+  // block's vectors, else by the first four waves
+  constexpr int LOADERS = (TOK * 8) % THREADS == 0 ? THREADS : 256;
+  constexpr int XL = TOK * 8 / LOADERS;       // token loads of a loading lane per step (LOADERS / 8 rows each)
+  static_assert(XL >= 1 && XL * LOADERS == TOK * 8 && LOADERS <= THREADS, "whole loads");
   __shared__ b128 ws[GW][32 * 8];            // per wave: one step of its 32 weight rows x 8 vectors
   __shared__ int red[GW];
   __shared__ int home[2];
@@ -1855,7 +1859,8 @@ __global__ __launch_bounds__(64 * GW, GW == 8 ? 1 : TJ <= 2 ? MOE_A2A_GEMM_OCC :
       wslot[i] = row * 8 + slot;
       if (i < 2) wpast[i] = vec >= tail_vecs ? OUT_OF_RANGE : 0;  // (loads i and i + 2 take the same vector)
     }
-    constexpr int XROWS = THREADS / 8;  // token rows one load of the workgroup covers: 32 or 64
+    constexpr int XROWS = LOADERS / 8;  // token rows one load of the workgroup covers: 32 or 64
+    const bool loader = LOADERS == THREADS || tid < LOADERS;  // (whole waves)
     const int xrow = tid >> 3, xvec = slot ^ ((xrow >> 1) & 7);  // (XROWS * i does not change bits 1..3)
     const int xpast = xvec >= tail_vecs ? OUT_OF_RANGE : 0;
 #pragma unroll
@@ -1878,14 +1883,14 @@ __global__ __launch_bounds__(64 * GW, GW == 8 ? 1 : TJ <= 2 ? MOE_A2A_GEMM_OCC :
       // issued nor parked, and a tile of 32 tokens without one is not multiplied)
 #pragma unroll
       for (int i = 0; i < XL; ++i)
-        if (i * XROWS < live)
+        if (loader && i * XROWS < live)
           xv[set][i] = __builtin_amdgcn_raw_buffer_load_b128(xbuf, xoff[i] + (last ? xpast : 0),
                                                              at * (GEMM_KSTEP * 2), 0);
     };
     auto park_x = [&](int set) {
 #pragma unroll
       for (int i = 0; i < XL; ++i)
-        if (i * XROWS < live) xs[set][tid + THREADS * i] = xv[set][i];
+        if (loader && i * XROWS < live) xs[set][tid + LOADERS * i] = xv[set][i];
     };
     auto compute = [&](int set) {
 #pragma unroll
@@ -2920,13 +2925,28 @@ int launch_grouped_gemm(const void* x, const int32_t* rows_of_group, const void*
   const int tj = rows_hint > (long long)MOE_A2A_GEMM_ROWS_FOR_128 * groups ? 4 : 2;
   // every group can end in a partly filled block of tokens; the kernel strides over what the hint misses
   const long long row_blocks = rows_hint / (tj * 32) + groups;
-  // Workgroups of 256 columns (8 waves) pull an expert's token rows through half as many L1s as
-  // workgroups of 128; taken when blocks hold 128 tokens and there are still tiles for every unit.
+  // Workgroups of up to 256 columns (8 waves, one workgroup per compute unit) pull an expert's
+  // token rows through half as many L1s as workgroups of 128; taken when blocks hold 128 tokens and
+  // there are tiles for every unit. One workgroup per unit makes the launch a number of rounds over
+  // the units, and half a round at the end leaves half the chip idle (measured: 0.66 of HBM peak at
+  // 3.5 rounds, 0.71 at 7.0), so the width is the widest of 8..5 waves whose last round is nearly
+  // full, judged from the blocks the row count promises (every group at least one).
 #ifndef MOE_A2A_GEMM_WIDE_MIN_TILES
 #define MOE_A2A_GEMM_WIDE_MIN_TILES 512
 #endif
-  const bool wide = tj == 4 && row_blocks * ((N + 255) / 256) >= MOE_A2A_GEMM_WIDE_MIN_TILES;
-  const int cols = wide ? 256 : GEMM_COLS;
+  constexpr int UNITS = 256;  // compute units of an MI355X
+  int gw = 4;
+  if (tj == 4 && row_blocks * ((N + 255) / 256) >= MOE_A2A_GEMM_WIDE_MIN_TILES) {
+    const long long blocks = std::max<long long>(groups, (rows_hint + 127) / 128);
+    double best = -1.0;
+    for (int w = 8; w >= 5; --w) {
+      const long long tiles = blocks * ((N + 32 * w - 1) / (32 * w));
+      const double rounds = (double)tiles / UNITS, fill = rounds / std::ceil(rounds);
+      if (fill >= 0.95) { gw = w; break; }
+      if (fill > best) { best = fill; gw = w; }
+    }
+  }
+  const int cols = 32 * gw;
   const int col_tiles = (N + cols - 1) / cols;
   if ((max_rows / 64 + 1) * groups * col_tiles > INT_MAX / 2) return MOE_A2A_EINVAL;
   const int grid = mover_blocks(row_blocks * col_tiles);
@@ -2934,15 +2954,18 @@ int launch_grouped_gemm(const void* x, const int32_t* rows_of_group, const void*
   expert_gemm_kernel<DT, TJ, GW><<<grid, 64 * GW, 0, st>>>((const b128*)x, rows_of_group, (const b128*)w, \
                                                            (const uint16_t*)bias, (uint16_t*)y, groups,  \
                                                            (int)max_rows, N, K, col_tiles)
-  if (dtype == MOE_A2A_BF16) {
-    if (tj == 2) LAUNCH_G(MOE_A2A_BF16, 2, 4);
-    else if (wide) LAUNCH_G(MOE_A2A_BF16, 4, 8);
-    else LAUNCH_G(MOE_A2A_BF16, 4, 4);
-  } else {
-    if (tj == 2) LAUNCH_G(MOE_A2A_F16, 2, 4);
-    else if (wide) LAUNCH_G(MOE_A2A_F16, 4, 8);
-    else LAUNCH_G(MOE_A2A_F16, 4, 4);
-  }
+#define LAUNCH_GW(DT)                                 \
+  do {                                                \
+    if (tj == 2) LAUNCH_G(DT, 2, 4);                  \
+    else if (gw == 8) LAUNCH_G(DT, 4, 8);             \
+    else if (gw == 7) LAUNCH_G(DT, 4, 7);             \
+    else if (gw == 6) LAUNCH_G(DT, 4, 6);             \
+    else if (gw == 5) LAUNCH_G(DT, 4, 5);             \
+    else LAUNCH_G(DT, 4, 4);                          \
+  } while (0)
+  if (dtype == MOE_A2A_BF16) LAUNCH_GW(MOE_A2A_BF16);
+  else LAUNCH_GW(MOE_A2A_F16);
+#undef LAUNCH_GW
 #undef LAUNCH_G
   return launch_status();
 }
