@@ -1698,8 +1698,9 @@ __global__ __launch_bounds__(64 * ROWS) void expert_scale_wave_kernel(
 //
 // With a few dozen rows per expert the problem is bound by streaming the weights (C4: 3.3 GB of
 // them for 0.2 PFLOP), so the kernel is built to keep weight bytes in flight and to ask for them in
-// whole cache lines. A workgroup of 4 waves owns 128 output columns x one block of TJ*32 tokens of
-// one expert; a wave owns 32 of the columns for all tokens of the block (TJ tiles of
+// whole cache lines. A workgroup of GW waves (4, or 5 to 8 for blocks of 128 tokens) owns GW * 32
+// output columns x one block of TJ*32 tokens of one expert; a wave owns 32 of the columns for all
+// tokens of the block (TJ tiles of
 // v_mfma_f32_32x32x16, fp32 accumulators in registers) and walks the input dimension 64 elements
 // (128 bytes of every row) at a time.
 //
@@ -1708,8 +1709,8 @@ __global__ __launch_bounds__(64 * ROWS) void expert_scale_wave_kernel(
 // TB/s against 5.6 with the same bytes requested line by line). So a wave loads its 32 x 128 bytes
 // of a step with 8 lanes per line, drops them into 4 KB of LDS of its own, and picks the operands
 // up from there in MFMA layout. No barrier is involved: a wave's LDS operations execute in order.
-// Tokens: the rows of the block are what the 4 waves share. Each step's 128 bytes of every token
-// are loaded once per workgroup, parked in LDS and read from there by all four: one LDS barrier per
+// Tokens: the rows of the block are what the waves share. Each step's 128 bytes of every token
+// are loaded once per workgroup, parked in LDS and read from there by all of them: one LDS barrier per
 // step. Both kinds of loads are issued DEPTH steps ahead of their use; the vector memory counter
 // retires in order, so the token loads run one step ahead of the weights: waiting for the tokens
 // that are parked next never waits for the weights issued after them.

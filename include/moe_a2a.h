@@ -324,7 +324,9 @@ int moe_a2a_expert_scale(const moe_a2a_shape* shape, const void* expert_x,
  *   expert_y   [nle, max_recv, H] out; rows at or past expert_num_tokens[le] are
  *              not written
  * Rows are processed in blocks of 64 or 128 tokens found from the device-side
- * counts, so the work follows the rows, not the experts. Limits: hidden_dim a
+ * counts, so the work follows the rows, not the experts; with blocks of 128
+ * tokens a workgroup is 160 to 256 columns wide, the width picked from
+ * rows_hint so that the launch fills the compute units in whole rounds. Limits: hidden_dim a
  * multiple of 32, all three buffers 16-byte aligned (MOE_A2A_EINVAL / EALIGN).
  * Sums are formed in float32 in the order of the matrix unit, which is not the
  * order of a CPU matmul: results lie within what float32 accumulation in any
@@ -354,6 +356,9 @@ int moe_a2a_expert_gemm(const moe_a2a_shape* shape, const void* expert_x,
  * order); otherwise the kernel of moe_a2a_expert_gemm with one group of m rows.
  * Limits: n a multiple of 32, k a multiple of 8, input / weight / output 16-byte
  * and bias 8-byte aligned (MOE_A2A_EINVAL / EALIGN). m == 0 is a no-op.
+ * The first call on a GPU that takes the first of the three kernels sets a kernel
+ * attribute (it uses more LDS than a kernel gets by default): make that call
+ * outside a graph capture.
  * The reduce-scatter that follows in the reference (gemm-rs/reference.py:58-59)
  * is an exchange between GPUs and not part of this library.
  */
