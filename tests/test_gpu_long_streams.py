@@ -173,3 +173,65 @@ def test_graph_replays_of_the_long_stream_step():
         graph.replay()
         torch.cuda.synchronize()
         assert torch.equal(y[: d0.num_tokens], eager[0]), f"replay {i}"
+
+
+def test_counts_beyond_capacity_are_cut_off_by_the_long_stream_entry_points():
+    """Device-side counts that claim more rows than the caller says its buffers hold, through the
+    C ABI: the planner, the table builder and the movers stop at the stated capacity, whatever the
+    hint. Tensors are allocated with 64 rows and pre-filled with a sentinel; the calls are told 24."""
+    import ctypes as C
+    from amd_distributed_2025_amd import HIPAllToAll, _lib
+    from amd_distributed_2025_amd.task import MoEConfig
+    from oracle import moe_a2a_oracle as orc
+    from tests.test_gpu_parity import valid_rows
+
+    W, nle, K, H, max_T = 4, 2, 2, 72, 32
+    cfg = MoEConfig(W * nle, K, H, max_T, in_dtype=torch.bfloat16, out_dtype=torch.bfloat16)
+    a = HIPAllToAll(cfg, 0, W, device=DEV)
+    max_recv = max_T * W
+    rng = np.random.default_rng(78)
+    ALLOC, CAP, SENT = 64, 24, -12345
+    p = lambda t: C.c_void_p(t.data_ptr())
+    st = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    shape = C.byref(a.shape)
+    meta_np = np.zeros((ALLOC, 5), np.int32)
+    meta_np[:, 0] = rng.integers(0, nle, ALLOC)
+    meta_np[:, 1] = np.minimum(np.arange(ALLOC) // 10, W - 1)
+    pairs = rng.permutation(max_T * K)[:ALLOC]          # every (token, k) at most once
+    meta_np[:, 2], meta_np[:, 3] = pairs // K, pairs % K
+    recv_buf = torch.from_numpy(rng.integers(0, 0x4400, (ALLOC, H), dtype=np.int16)).view(torch.bfloat16).to(DEV)
+    recv_meta = torch.from_numpy(meta_np).to(DEV)
+    counts40 = torch.tensor([10, 10, 10, 10], dtype=torch.int32, device=DEV)
+
+    num = torch.full((nle,), SENT, dtype=torch.int32, device=DEV)
+    ex = torch.zeros(nle, max_recv, H, dtype=torch.bfloat16, device=DEV)
+    em = torch.full((nle, max_recv, 5), SENT, dtype=torch.int32, device=DEV)
+    pos = torch.full((ALLOC,), SENT, dtype=torch.int32, device=DEV)
+    for hint in (0, 7, CAP, 40, 1000):
+        num.fill_(SENT); em.fill_(SENT); pos.fill_(SENT)
+        _lib.call("moe_a2a_dispatch_recv_long", shape, p(recv_buf), p(recv_meta), p(counts40), hint, CAP,
+                  p(num), p(ex), p(em), None, p(pos), st)
+        torch.cuda.synchronize()
+        cnt, local, where, order = orc.expert_placement(meta_np[:CAP], nle)
+        assert np.array_equal(num.cpu().numpy(), cnt), hint
+        assert np.array_equal(valid_rows(em, cnt).numpy(), meta_np[:CAP][order]), hint
+        assert np.array_equal(bits(valid_rows(ex, cnt)), bits(recv_buf[:CAP])[order]), hint
+        assert bool((pos[CAP:] == SENT).all()), hint          # the planner wrote no position past the capacity
+        for le in range(nle):
+            assert bool((em[le, int(cnt[le]):] == SENT).all()), hint
+
+    weights = torch.from_numpy(rng.random((max_T, K), dtype=np.float32)).to(DEV)
+    y = torch.zeros(max_T, H, dtype=torch.bfloat16, device=DEV)
+    table = torch.full((max_T * K,), 63, dtype=torch.int32, device=DEV)  # stale entries that name a row past the capacity
+    for hint in (0, CAP, 40, 1000):
+        _lib.call("moe_a2a_combine_recv_long", shape, p(recv_buf), p(recv_meta), p(counts40), hint, CAP,
+                  p(weights), max_T, p(y), 0, _lib.BF16, p(table), st)
+        torch.cuda.synchronize()
+        want = orc.combine_recv(bits(recv_buf[:CAP]), meta_np[:CAP], weights.cpu().numpy(), max_T, "bf16")
+        assert np.array_equal(bits(y), want), hint
+    # null workspaces are refused before anything is launched
+    lib = _lib.load()
+    assert lib.moe_a2a_dispatch_recv_long(shape, p(recv_buf), p(recv_meta), p(counts40), CAP, CAP, p(num), p(ex), p(em),
+                                          None, None, st) == -1
+    assert lib.moe_a2a_combine_recv_long(shape, p(recv_buf), p(recv_meta), p(counts40), CAP, CAP, p(weights), max_T,
+                                         p(y), 0, _lib.BF16, None, st) == -1
