@@ -190,3 +190,37 @@ def test_unsupported_shapes_raise():
         a.expert_gemm(ex, torch.tensor([4], dtype=torch.int32, device=DEV), w)
     with pytest.raises(ValueError, match="weights must be"):
         a.expert_gemm(ex, torch.tensor([4], dtype=torch.int32, device=DEV), w[:, :64])
+
+
+@pytest.mark.parametrize("H,width", [(576, 5), (640, 6), (704, 7), (832, 8)])
+def test_wide_workgroups_of_every_width(H, width):
+    """With blocks of 128 tokens and many tiles a workgroup is 5 to 8 waves wide, the width picked
+    from the row count so that the launch fills the compute units in whole rounds: 128 experts of
+    about 60 rows and these four row lengths take the four widths (5 to 7 waves leave the token
+    loads to the first four). Signed permutation weights: exact."""
+    print(f"wide workgroups: H={H}, expected width {width} waves", flush=True)
+    dt, nle, max_tokens = torch.bfloat16, 128, 140
+    rng = np.random.default_rng(H)
+    a, cfg = rank_object(1, nle, H, max_tokens, dt)
+    counts = [60] * nle
+    for i, c in enumerate([0, 140, 1, 129, 128, 127, 33]):   # ragged, and the total stays 60 * nle
+        counts[i], counts[nle - 1 - i] = c, 120 - c if c <= 120 else 0
+    counts[1], counts[nle - 2] = 140, 0
+    total = 60 * nle
+    counts[nle // 2] += total - sum(counts)
+    assert sum(counts) == total and 0 <= min(counts) and max(counts) <= max_tokens
+    xb = rng.integers(0, 1 << 16, (nle, max_tokens, H), dtype=np.uint16)
+    xb[~np.isfinite(orc.b16_to_f32(xb, "bf16"))] = 0x3C00
+    perm = np.stack([rng.permutation(H) for _ in range(nle)])
+    sign = rng.choice([-1.0, 1.0], (nle, H))
+    w = torch.zeros(nle, H, H, dtype=dt)
+    for le in range(nle):
+        w[le, torch.arange(H), torch.from_numpy(perm[le])] = torch.from_numpy(sign[le]).to(dt)
+    got = run_gemm(a, from_bits(xb, dt).to(DEV), counts, w.to(DEV), hint=total)
+    check_padding_untouched(got, counts)
+    for le, c in enumerate(counts):
+        moved = xb[le, :c][:, perm[le]]
+        want = np.where(sign[le] < 0, moved ^ 0x8000, moved).astype(np.uint16)
+        zero = (want & 0x7FFF) == 0
+        assert np.array_equal(got[le, :c][~zero], want[~zero]), f"expert {le}"
+        assert ((got[le, :c][zero] & 0x7FFF) == 0).all()
