@@ -2227,18 +2227,31 @@ __global__ __launch_bounds__(64 * WM * WN) void dense_gemm_kernel(
   __syncthreads();
   read_frags(0, 0, 0);
   // One memory instruction between two MFMAs: a wave that issues its loads or stores back to back
-  // waits for the queues of the memory pipes and issues no MFMA meanwhile.
-#define MOE_A2A_INTERLEAVE()                                          \
-  _Pragma("unroll") for (int q = 0; q < 4; ++q) {                     \
-    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                \
-    __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);                \
-    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                \
-    __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);                \
-    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                \
-    __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);                \
-    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                \
-    __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);                \
-  }                                                                   \
+  // waits for the queues of the memory pipes and issues no MFMA meanwhile. A slice holds TM * TN
+  // MFMAs, TM + TN fragment reads and one quarter's stores and loads; the 256 x 256 tile has its
+  // measured order (read, store, read, load), smaller tiles spread theirs over the leading MFMAs.
+  constexpr int N_MFMA = TM * TN, N_QUARTER = (LA > LB ? LA : LB) / 2;
+  constexpr int READS_EACH = (TM + TN + N_MFMA - 1) / N_MFMA, MOVES_EACH = (N_QUARTER + N_MFMA - 1) / N_MFMA;
+#define MOE_A2A_INTERLEAVE()                                            \
+  if constexpr (N_MFMA == 16 && N_QUARTER == 4) {                       \
+    _Pragma("unroll") for (int q = 0; q < 4; ++q) {                     \
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                \
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);                \
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                \
+      __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);                \
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                \
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);                \
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                \
+      __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);                \
+    }                                                                   \
+  } else {                                                              \
+    _Pragma("unroll") for (int q = 0; q < N_MFMA; ++q) {                \
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                \
+      __builtin_amdgcn_sched_group_barrier(0x100, READS_EACH, 0);       \
+      __builtin_amdgcn_sched_group_barrier(0x200, MOVES_EACH, 0);       \
+      __builtin_amdgcn_sched_group_barrier(0x020, MOVES_EACH, 0);       \
+    }                                                                   \
+  }                                                                     \
   __builtin_amdgcn_sched_barrier(0);
   auto one_step = [&](int step, int cur) {  // cur = step & 1, a constant where this is called
     read_frags(1, cur, 1);
@@ -2971,45 +2984,89 @@ int launch_grouped_gemm(const void* x, const int32_t* rows_of_group, const void*
   return launch_status();
 }
 
-#ifndef MOE_A2A_DENSE_MIN_TILES
-#define MOE_A2A_DENSE_MIN_TILES 128  // 256 x 256 tiles of the output from which the dense kernel is used
+#ifndef MOE_A2A_DENSE_MIN_ROWS
+#define MOE_A2A_DENSE_MIN_ROWS 33  // rows from which the dense kernel is used
 #endif
-constexpr int MOE_A2A_NOT_DENSE = 1;  // (internal) the shape is left to the grouped kernel
+#ifndef MOE_A2A_DENSE_TILE
+#define MOE_A2A_DENSE_TILE 0  // (measurements) 256, 128 or 64: that tile height for every shape
+#endif
+constexpr int MOE_A2A_NOT_DENSE = 1;  // (internal) the shape is left to the next kernel
 
-// The dense kernel for products with enough 256 x 256 tiles to fill the chip; MOE_A2A_NOT_DENSE
-// otherwise (few rows: the grouped kernel, which is built for streaming the weights).
+// Which tile the dense kernel uses for an M x N x K product: 256 x 256 (one workgroup per compute
+// unit, the highest rate per unit once every unit has work for several tiles), 128 x 128 (two
+// workgroups per unit, about 0.8 of that rate, but four times the tiles: fuller last round, and
+// one workgroup's prologue and epilogue overlap the other's MFMAs, which decides short K) or
+// 64 x 128 (for outputs that even 128 x 128 tiles cannot spread over the 256 units).
+// The costs are in units of a 128 x 128 tile's work at the big tile's rate; the constants are
+// fits to measurements on an MI355X (rows 64 .. 8192, K 256 .. 4608).
+int dense_tile_rows(long long M, long long N, int K) {
+  if (MOE_A2A_DENSE_TILE) return MOE_A2A_DENSE_TILE;
+  constexpr double UNITS = 256.0;
+  const double steps = (K + GEMM_KSTEP - 1) / GEMM_KSTEP;
+  const double big = (double)((M + 255) / 256) * (double)((N + 255) / 256);
+  const double mid = (double)((M + 127) / 128) * (double)((N + 127) / 128);
+  const double low = (double)((M + 63) / 64) * (double)((N + 127) / 128);
+  if (low <= UNITS) return 64;
+  // a last round that is partly empty costs about half of what it leaves idle (the busy units
+  // run faster meanwhile); per tile, fixed work worth 3 steps (big) and 1 step (mid)
+  const double big_cost = 4.0 * 0.5 * (big / UNITS + ceil(big / UNITS)) * (steps + 3.0) / steps;
+  const double mid_cost = 1.25 * fmax(mid / UNITS, 1.0) * (steps + 1.0) / steps;
+  return big_cost <= mid_cost ? 256 : 128;
+}
+
+constexpr size_t dense_lds_bytes(int BM, int BN) { return 2 * (size_t)(BM + BN) * 8 * sizeof(b128); }
+
+// The tile buffers can be more LDS than a kernel gets by default: allowed once per GPU, for every
+// tile and type at once, so that only the first dense call on a GPU touches kernel attributes.
+int allow_dense_lds() {
+  static bool allowed[MAX_GPUS] = {};
+  int gpu = -1;
+  if (hipGetDevice(&gpu) != hipSuccess || gpu < 0 || gpu >= MAX_GPUS) return MOE_A2A_ELAUNCH;
+  std::lock_guard<std::mutex> lock(static_plan_mutex);
+  if (allowed[gpu]) return MOE_A2A_OK;
+  bool ok = true;
+  auto allow = [&](const void* kernel, size_t bytes) {
+    ok = ok && hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes) == hipSuccess;
+  };
+  allow((const void*)dense_gemm_kernel<MOE_A2A_BF16, 2, 2, 4, 4>, dense_lds_bytes(256, 256));
+  allow((const void*)dense_gemm_kernel<MOE_A2A_F16, 2, 2, 4, 4>, dense_lds_bytes(256, 256));
+  allow((const void*)dense_gemm_kernel<MOE_A2A_BF16, 2, 2, 2, 2>, dense_lds_bytes(128, 128));
+  allow((const void*)dense_gemm_kernel<MOE_A2A_F16, 2, 2, 2, 2>, dense_lds_bytes(128, 128));
+  allow((const void*)dense_gemm_kernel<MOE_A2A_BF16, 2, 2, 1, 2>, dense_lds_bytes(64, 128));
+  allow((const void*)dense_gemm_kernel<MOE_A2A_F16, 2, 2, 1, 2>, dense_lds_bytes(64, 128));
+  if (!ok) return MOE_A2A_ELAUNCH;
+  allowed[gpu] = true;
+  return MOE_A2A_OK;
+}
+
+// The dense kernel for products of more than a few rows; MOE_A2A_NOT_DENSE otherwise (the kernels
+// that split K over the waves of a workgroup or stream the weights once).
 int launch_dense_gemm(const void* a, const void* b, const void* bias, void* c, int M, int N, int K,
                       int dtype, hipStream_t st) {
   if (dtype != MOE_A2A_F16 && dtype != MOE_A2A_BF16) return MOE_A2A_EINVAL;
   if (N % 32 != 0 || K % 8 != 0) return MOE_A2A_EINVAL;
   if (!all_aligned(16, a, b, c) || !all_aligned(8, bias)) return MOE_A2A_EALIGN;
-  constexpr int BM = 256, BN = 256;
-  const long long tiles_m = ((long long)M + BM - 1) / BM, tiles_n = ((long long)N + BN - 1) / BN;
-  if (tiles_m * tiles_n < MOE_A2A_DENSE_MIN_TILES || tiles_m * tiles_n > INT_MAX / 2) return MOE_A2A_NOT_DENSE;
+  if (M < MOE_A2A_DENSE_MIN_ROWS) return MOE_A2A_NOT_DENSE;
   if ((long long)K * 2 * 256 >= (1 << 30)) return MOE_A2A_NOT_DENSE;  // 32-bit byte offsets inside a tile's rows
-  constexpr size_t lds_bytes = 2 * (BM + BN) * 8 * sizeof(b128);
+  const int tile = dense_tile_rows(M, N, K);
+  const int BM = tile, BN = tile == 64 ? 128 : tile;
+  const long long tiles_m = ((long long)M + BM - 1) / BM, tiles_n = ((long long)N + BN - 1) / BN;
+  if (tiles_m * tiles_n > INT_MAX / 2) return MOE_A2A_NOT_DENSE;
+  const size_t lds_bytes = dense_lds_bytes(BM, BN);
   const int grid = (int)(tiles_m * tiles_n);
-  // the tile buffers are more LDS than a kernel gets by default: allowed once per GPU and kernel
-  int gpu = -1;
-  if (hipGetDevice(&gpu) != hipSuccess || gpu < 0 || gpu >= MAX_GPUS) return MOE_A2A_ELAUNCH;
-#define LAUNCH_D(DT)                                                                              \
-  do {                                                                                            \
-    auto kernel = dense_gemm_kernel<DT, 2, 2, 4, 4>;                                              \
-    static bool allowed[MAX_GPUS] = {};                                                           \
-    {                                                                                             \
-      std::lock_guard<std::mutex> lock(static_plan_mutex);                                        \
-      if (!allowed[gpu]) {                                                                        \
-        if (hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize,  \
-                                (int)lds_bytes) != hipSuccess)                                    \
-          return MOE_A2A_ELAUNCH;                                                                 \
-        allowed[gpu] = true;                                                                      \
-      }                                                                                           \
-    }                                                                                             \
-    kernel<<<grid, 256, lds_bytes, st>>>((const b128*)a, (const b128*)b, (const uint16_t*)bias,   \
-                                         (uint16_t*)c, M, N, K, (int)tiles_m, (int)tiles_n);      \
+  if (const int rc = allow_dense_lds()) return rc;
+#define LAUNCH_D(DT, TM, TN)                                                             \
+  dense_gemm_kernel<DT, 2, 2, TM, TN><<<grid, 256, lds_bytes, st>>>(                     \
+      (const b128*)a, (const b128*)b, (const uint16_t*)bias, (uint16_t*)c, M, N, K, (int)tiles_m, (int)tiles_n)
+#define LAUNCH_DT(DT)                         \
+  do {                                        \
+    if (tile == 256) LAUNCH_D(DT, 4, 4);      \
+    else if (tile == 128) LAUNCH_D(DT, 2, 2); \
+    else LAUNCH_D(DT, 1, 2);                  \
   } while (0)
-  if (dtype == MOE_A2A_BF16) LAUNCH_D(MOE_A2A_BF16);
-  else LAUNCH_D(MOE_A2A_F16);
+  if (dtype == MOE_A2A_BF16) LAUNCH_DT(MOE_A2A_BF16);
+  else LAUNCH_DT(MOE_A2A_F16);
+#undef LAUNCH_DT
 #undef LAUNCH_D
   return launch_status();
 }
@@ -3018,32 +3075,25 @@ int launch_dense_gemm(const void* a, const void* b, const void* bias, void* c, i
 #define MOE_A2A_SKINNY_MAX_TILES 192  // tiles of 128 columns below which K is split inside the workgroup
 #endif
 
-// Products whose tiles of 128 columns would leave compute units idle: 32 columns per workgroup,
-// K split over its waves. MOE_A2A_NOT_DENSE when the grouped kernel is the better fit.
+// Products of at most 64 rows whose tiles of 128 columns would leave compute units idle: 32
+// columns per workgroup, K split over its waves. MOE_A2A_NOT_DENSE when the grouped kernel is
+// the better fit.
 int launch_skinny_gemm(const void* x, const void* w, const void* bias, void* y, int M, int N, int K,
                        int dtype, hipStream_t st) {
   if (dtype != MOE_A2A_F16 && dtype != MOE_A2A_BF16) return MOE_A2A_EINVAL;
   if (N % 32 != 0 || K % 8 != 0) return MOE_A2A_EINVAL;
   if (!all_aligned(16, x, w, y) || !all_aligned(8, bias)) return MOE_A2A_EALIGN;
-  if ((long long)K * 2 * 128 >= (1 << 30)) return MOE_A2A_NOT_DENSE;
-  const int tj = M > 64 ? 4 : 2;
-  const long long row_blocks = ((long long)M + tj * 32 - 1) / (tj * 32);
-  const long long wide_tiles = row_blocks * ((N + GEMM_COLS - 1) / GEMM_COLS);
+  if (M > 64 || (long long)K * 2 * 128 >= (1 << 30)) return MOE_A2A_NOT_DENSE;
+  const int wide_tiles = (N + GEMM_COLS - 1) / GEMM_COLS;
   const int steps = (K + GEMM_KSTEP - 1) / GEMM_KSTEP;
   if (wide_tiles >= MOE_A2A_SKINNY_MAX_TILES || steps < 2 * NWAVES) return MOE_A2A_NOT_DENSE;
-  const long long grid = row_blocks * (N / 32);
-  if (grid > INT_MAX / 2) return MOE_A2A_NOT_DENSE;
-#define LAUNCH_K(DT, TJ)                                                                           \
-  skinny_gemm_kernel<DT, TJ><<<(int)grid, BLOCK, 0, st>>>((const b128*)x, (const b128*)w,         \
-                                                          (const uint16_t*)bias, (uint16_t*)y, M, N, K, N / 32)
-  if (dtype == MOE_A2A_BF16) {
-    if (tj == 2) LAUNCH_K(MOE_A2A_BF16, 2);
-    else LAUNCH_K(MOE_A2A_BF16, 4);
-  } else {
-    if (tj == 2) LAUNCH_K(MOE_A2A_F16, 2);
-    else LAUNCH_K(MOE_A2A_F16, 4);
-  }
-#undef LAUNCH_K
+  const int grid = N / 32;
+  if (dtype == MOE_A2A_BF16)
+    skinny_gemm_kernel<MOE_A2A_BF16, 2><<<grid, BLOCK, 0, st>>>(
+        (const b128*)x, (const b128*)w, (const uint16_t*)bias, (uint16_t*)y, M, N, K, N / 32);
+  else
+    skinny_gemm_kernel<MOE_A2A_F16, 2><<<grid, BLOCK, 0, st>>>(
+        (const b128*)x, (const b128*)w, (const uint16_t*)bias, (uint16_t*)y, M, N, K, N / 32);
   return launch_status();
 }
 

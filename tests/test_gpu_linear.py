@@ -63,12 +63,15 @@ def test_task_shapes(m, n, k, has_bias, seed):
 
 
 @pytest.mark.parametrize("dt", [torch.bfloat16, torch.float16], ids=["bf16", "fp16"])
-# (the last four: few rows and many steps of K, where a workgroup's waves split K among them)
-@pytest.mark.parametrize("m,n,k", [(1, 32, 8), (70, 96, 72), (129, 160, 360), (300, 2880, 200), (64, 64, 64),
-                                   (1, 32, 512), (64, 96, 520), (70, 64, 1000), (200, 160, 1096),
-                                   # many rows: tiles of 256 x 256 with ragged last tiles in both directions,
-                                   # one and several steps of K, a K tail
-                                   (3000, 2944, 72), (2050, 4128, 200), (4100, 2080, 8)])
+# up to 64 rows: with many steps of K a workgroup's waves split K among them, else the grouped kernel
+@pytest.mark.parametrize("m,n,k", [(1, 32, 8), (64, 64, 64), (1, 32, 512), (64, 96, 520), (33, 2880, 1000),
+                                   # from 65 rows: tiles of 64 x 128 (outputs that fill few compute units) ...
+                                   (65, 64, 520), (70, 96, 72), (129, 160, 360), (300, 2880, 200), (70, 64, 1000),
+                                   (200, 160, 1096),
+                                   # ... of 128 x 128 (short K, or too few tiles of 256 x 256 for every unit) ...
+                                   (3000, 2944, 72), (2050, 4128, 200), (4100, 2080, 8), (1000, 4128, 1096),
+                                   # ... and of 256 x 256; ragged last tiles in both directions and a K tail each
+                                   (3900, 4000, 1032)])
 def test_small_integers_with_bias_are_exact(m, n, k, dt):
     print(f"linear integers m={m} n={n} k={k} {dt}", flush=True)
     rng = np.random.default_rng(m * n + k)
@@ -84,12 +87,13 @@ def test_small_integers_with_bias_are_exact(m, n, k, dt):
     out = torch.full((m + 2, n), 777.0, dtype=dt, device=DEV)
     gemm_rs.local_product((pad[1:m + 1], wpad[1:n + 1], bias), out=out[1:m + 1])
     torch.cuda.synchronize()
-    want = x @ w.T + b[None, :]
-    assert np.abs(want).max() <= 256 and np.abs(x @ w.T).max() <= 256  # integers both 16-bit types hold
+    prod = (x.astype(np.float64) @ w.T.astype(np.float64)).astype(np.int64)  # exact: small integers
+    want = prod + b[None, :]
+    assert np.abs(want).max() <= 256 and np.abs(prod).max() <= 256  # integers both 16-bit types hold
     assert np.array_equal(out[1:m + 1].float().cpu().numpy(), want.astype(np.float32))
     assert (out[0] == 777.0).all() and (out[m + 1] == 777.0).all()
     no_bias = gemm_rs.local_product((pad[1:m + 1], wpad[1:n + 1], None))
-    assert np.array_equal(no_bias.float().cpu().numpy(), (x @ w.T).astype(np.float32))
+    assert np.array_equal(no_bias.float().cpu().numpy(), prod.astype(np.float32))
 
 
 def test_bias_is_added_to_the_rounded_product():
