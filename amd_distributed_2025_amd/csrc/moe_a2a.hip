@@ -1973,22 +1973,24 @@ __global__ __launch_bounds__(64 * GW, GW > 4 ? 1 : TJ <= 2 ? MOE_A2A_GEMM_OCC : 
 
 // ---------------------------------------------------------------- product with few rows
 //
-// Y[M, N] = X[M, K] @ W[N, K]^T with so few rows that tiles of 128 columns do not fill the chip
-// (M = 64, N = 7168: 56 workgroups). Here a workgroup owns only 32 output columns x one block of
-// tokens, and its four waves split K: wave w takes steps w, w + 4, ... of 64 elements, streams
+// Y[M, N] = X[M, K] @ W[N, K]^T for at most 64 rows: the weights are streamed once and no tile
+// shape gives every compute unit work (M = 64, N = 7168: 56 tiles of 128 columns). Here a
+// workgroup owns only 32 output columns x one block of 32 or 64 tokens, and its KW waves (four,
+// eight for long K) split K: wave w takes steps w, w + KW, ... of 64 elements, streams
 // its own slices of the 32 weight rows and of the token rows (both 8 lanes per 128-byte line,
 // turned into MFMA layout through LDS private to the wave: no barrier in the loop), and keeps
 // partial sums in registers. At the end the partial sums meet in LDS and are added in a fixed
-// order (wave 0 + 1 + 2 + 3), so results do not depend on scheduling.
+// order (wave 0 + 1 + 2 + ...), so results do not depend on scheduling.
 
-template <int DT, int TJ>
-__global__ __launch_bounds__(BLOCK, TJ <= 2 ? 3 : 2) void skinny_gemm_kernel(
+template <int DT, int TJ, int KW>
+__global__ __launch_bounds__(64 * KW) void skinny_gemm_kernel(
     const b128* __restrict__ X, const b128* __restrict__ Wt, const uint16_t* __restrict__ bias,
     uint16_t* __restrict__ Y, int M, int N, int K, int col_units) {
   constexpr int TOK = TJ * 32;
   constexpr int XL = TJ * 4;  // token loads per lane and step: TOK rows x 8 vectors over 64 lanes
-  __shared__ b128 wsl[NWAVES][32 * 8];
-  __shared__ b128 xsl[NWAVES][TOK * 8];
+  extern __shared__ b128 skinny_lds[];  // per wave: 32 weight rows, then TOK token rows, of 8 vectors
+  b128(*wsl)[32 * 8] = reinterpret_cast<b128(*)[32 * 8]>(skinny_lds);
+  b128(*xsl)[TOK * 8] = reinterpret_cast<b128(*)[TOK * 8]>(skinny_lds + KW * 32 * 8);
   const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
   const int row_vecs = K / 8, row_bytes = K * 2, steps = (K + GEMM_KSTEP - 1) / GEMM_KSTEP;
   const int tail_vecs = row_vecs - (steps - 1) * 8;
@@ -2044,12 +2046,12 @@ __global__ __launch_bounds__(BLOCK, TJ <= 2 ? 3 : 2) void skinny_gemm_kernel(
   };
 
   load(0, wave);
-  load(1, wave + NWAVES);
-  for (int s = wave; s < steps; s += 2 * NWAVES) {
+  load(1, wave + KW);
+  for (int s = wave; s < steps; s += 2 * KW) {
     compute(0);
-    load(0, s + 2 * NWAVES);
-    if (s + NWAVES < steps) compute(1);
-    load(1, s + 3 * NWAVES);
+    load(0, s + 2 * KW);
+    if (s + KW < steps) compute(1);
+    load(1, s + 3 * KW);
   }
 
   // partial sums to LDS (a wave's region holds exactly its TJ x 16 floats per lane), then wave j
@@ -2067,7 +2069,7 @@ __global__ __launch_bounds__(BLOCK, TJ <= 2 ? 3 : 2) void skinny_gemm_kernel(
     for (int e = 0; e < 16; ++e) {
       float sum = reinterpret_cast<const float*>(xsl[0])[(j * 16 + e) * 64 + lane];
 #pragma unroll
-      for (int w = 1; w < NWAVES; ++w)
+      for (int w = 1; w < KW; ++w)
         sum = __fadd_rn(sum, reinterpret_cast<const float*>(xsl[w])[(j * 16 + e) * 64 + lane]);
       c[e] = sum;
     }
@@ -2984,9 +2986,6 @@ int launch_grouped_gemm(const void* x, const int32_t* rows_of_group, const void*
   return launch_status();
 }
 
-#ifndef MOE_A2A_DENSE_MIN_ROWS
-#define MOE_A2A_DENSE_MIN_ROWS 33  // rows from which the dense kernel is used
-#endif
 #ifndef MOE_A2A_DENSE_TILE
 #define MOE_A2A_DENSE_TILE 0  // (measurements) 256, 128 or 64: that tile height for every shape
 #endif
@@ -3015,10 +3014,11 @@ int dense_tile_rows(long long M, long long N, int K) {
 }
 
 constexpr size_t dense_lds_bytes(int BM, int BN) { return 2 * (size_t)(BM + BN) * 8 * sizeof(b128); }
+constexpr size_t skinny_lds_bytes(int tj, int waves) { return (size_t)waves * (32 + 32 * tj) * 8 * sizeof(b128); }
 
 // The tile buffers can be more LDS than a kernel gets by default: allowed once per GPU, for every
 // tile and type at once, so that only the first dense call on a GPU touches kernel attributes.
-int allow_dense_lds() {
+int allow_large_lds() {
   static bool allowed[MAX_GPUS] = {};
   int gpu = -1;
   if (hipGetDevice(&gpu) != hipSuccess || gpu < 0 || gpu >= MAX_GPUS) return MOE_A2A_ELAUNCH;
@@ -3034,6 +3034,8 @@ int allow_dense_lds() {
   allow((const void*)dense_gemm_kernel<MOE_A2A_F16, 2, 2, 2, 2>, dense_lds_bytes(128, 128));
   allow((const void*)dense_gemm_kernel<MOE_A2A_BF16, 2, 2, 1, 2>, dense_lds_bytes(64, 128));
   allow((const void*)dense_gemm_kernel<MOE_A2A_F16, 2, 2, 1, 2>, dense_lds_bytes(64, 128));
+  allow((const void*)skinny_gemm_kernel<MOE_A2A_BF16, 2, 8>, skinny_lds_bytes(2, 8));
+  allow((const void*)skinny_gemm_kernel<MOE_A2A_F16, 2, 8>, skinny_lds_bytes(2, 8));
   if (!ok) return MOE_A2A_ELAUNCH;
   allowed[gpu] = true;
   return MOE_A2A_OK;
@@ -3046,7 +3048,6 @@ int launch_dense_gemm(const void* a, const void* b, const void* bias, void* c, i
   if (dtype != MOE_A2A_F16 && dtype != MOE_A2A_BF16) return MOE_A2A_EINVAL;
   if (N % 32 != 0 || K % 8 != 0) return MOE_A2A_EINVAL;
   if (!all_aligned(16, a, b, c) || !all_aligned(8, bias)) return MOE_A2A_EALIGN;
-  if (M < MOE_A2A_DENSE_MIN_ROWS) return MOE_A2A_NOT_DENSE;
   if ((long long)K * 2 * 256 >= (1 << 30)) return MOE_A2A_NOT_DENSE;  // 32-bit byte offsets inside a tile's rows
   const int tile = dense_tile_rows(M, N, K);
   const int BM = tile, BN = tile == 64 ? 128 : tile;
@@ -3054,7 +3055,7 @@ int launch_dense_gemm(const void* a, const void* b, const void* bias, void* c, i
   if (tiles_m * tiles_n > INT_MAX / 2) return MOE_A2A_NOT_DENSE;
   const size_t lds_bytes = dense_lds_bytes(BM, BN);
   const int grid = (int)(tiles_m * tiles_n);
-  if (const int rc = allow_dense_lds()) return rc;
+  if (const int rc = allow_large_lds()) return rc;
 #define LAUNCH_D(DT, TM, TN)                                                             \
   dense_gemm_kernel<DT, 2, 2, TM, TN><<<grid, 256, lds_bytes, st>>>(                     \
       (const b128*)a, (const b128*)b, (const uint16_t*)bias, (uint16_t*)c, M, N, K, (int)tiles_m, (int)tiles_n)
@@ -3071,6 +3072,9 @@ int launch_dense_gemm(const void* a, const void* b, const void* bias, void* c, i
   return launch_status();
 }
 
+#ifndef MOE_A2A_SKINNY_WAVES
+#define MOE_A2A_SKINNY_WAVES 0  // (measurements) 4 or 8: that many waves for every shape
+#endif
 #ifndef MOE_A2A_SKINNY_MAX_TILES
 #define MOE_A2A_SKINNY_MAX_TILES 192  // tiles of 128 columns below which K is split inside the workgroup
 #endif
@@ -3088,12 +3092,25 @@ int launch_skinny_gemm(const void* x, const void* w, const void* bias, void* y, 
   const int steps = (K + GEMM_KSTEP - 1) / GEMM_KSTEP;
   if (wide_tiles >= MOE_A2A_SKINNY_MAX_TILES || steps < 2 * NWAVES) return MOE_A2A_NOT_DENSE;
   const int grid = N / 32;
-  if (dtype == MOE_A2A_BF16)
-    skinny_gemm_kernel<MOE_A2A_BF16, 2><<<grid, BLOCK, 0, st>>>(
-        (const b128*)x, (const b128*)w, (const uint16_t*)bias, (uint16_t*)y, M, N, K, N / 32);
-  else
-    skinny_gemm_kernel<MOE_A2A_F16, 2><<<grid, BLOCK, 0, st>>>(
-        (const b128*)x, (const b128*)w, (const uint16_t*)bias, (uint16_t*)y, M, N, K, N / 32);
+  // eight waves keep more of the stream in flight (measured 10 to 13 % less time from 28 steps
+  // on); with few steps the four extra partial sums cost more than that
+  const int waves = MOE_A2A_SKINNY_WAVES ? MOE_A2A_SKINNY_WAVES : steps >= 24 ? 8 : 4;
+  const int tj = M <= 32 ? 1 : 2;
+  if (const int rc = allow_large_lds()) return rc;
+#define LAUNCH_K(DT, TJ, KW)                                                              \
+  skinny_gemm_kernel<DT, TJ, KW><<<grid, 64 * KW, skinny_lds_bytes(TJ, KW), st>>>(        \
+      (const b128*)x, (const b128*)w, (const uint16_t*)bias, (uint16_t*)y, M, N, K, N / 32)
+#define LAUNCH_KW(DT)                                      \
+  do {                                                     \
+    if (waves == 8 && tj == 2) LAUNCH_K(DT, 2, 8);         \
+    else if (waves == 8) LAUNCH_K(DT, 1, 8);               \
+    else if (tj == 2) LAUNCH_K(DT, 2, 4);                  \
+    else LAUNCH_K(DT, 1, 4);                               \
+  } while (0)
+  if (dtype == MOE_A2A_BF16) LAUNCH_KW(MOE_A2A_BF16);
+  else LAUNCH_KW(MOE_A2A_F16);
+#undef LAUNCH_KW
+#undef LAUNCH_K
   return launch_status();
 }
 
@@ -3116,10 +3133,10 @@ int moe_a2a_linear(const void* input, const void* weight, const void* bias, int3
                    int32_t k, int32_t dtype, void* output, void* stream) {
   if (m < 0 || n < 1 || k < 1 || !weight || (m > 0 && (!input || !output))) return MOE_A2A_EINVAL;
   if (m == 0) return MOE_A2A_OK;
-  const int dense = launch_dense_gemm(input, weight, bias, output, m, n, k, dtype, (hipStream_t)stream);
-  if (dense != MOE_A2A_NOT_DENSE) return dense;
   const int skinny = launch_skinny_gemm(input, weight, bias, output, m, n, k, dtype, (hipStream_t)stream);
   if (skinny != MOE_A2A_NOT_DENSE) return skinny;
+  const int dense = launch_dense_gemm(input, weight, bias, output, m, n, k, dtype, (hipStream_t)stream);
+  if (dense != MOE_A2A_NOT_DENSE) return dense;
   return launch_grouped_gemm(input, nullptr, weight, bias, output, 1, m, m, n, k, dtype,
                              (hipStream_t)stream);
 }

@@ -21,6 +21,15 @@ from . import _binding
 
 input_t = Tuple[torch.Tensor, torch.Tensor, Optional[torch.Tensor]]
 
+# (m, n, k of the 8-rank job, has_bias, seed): gemm-rs/task.yml:66-76 (tests) and :80-85 (benchmarks,
+# ranked by their geometric mean, task.yml:62)
+TASK_TESTS = [(64, 2880, 2880, True, 2035), (64, 3584, 14336, True, 13), (512, 3584, 14336, True, 4297),
+              (512, 4608, 36864, False, 1597), (2048, 4096, 7168, False, 716), (2048, 8192, 30720, False, 20201),
+              (4096, 2880, 2880, True, 136), (4096, 8192, 2048, True, 138), (8192, 3584, 14336, True, 748),
+              (8192, 4608, 36864, True, 4422), (8192, 8192, 28672, False, 1536)]
+TASK_BENCHMARKS = [(64, 7168, 18432, False, 1234), (512, 4096, 12288, True, 663), (2048, 2880, 2880, True, 166),
+                   (4096, 4096, 4096, False, 1371), (8192, 4096, 14336, True, 7168), (8192, 8192, 29568, False, 42)]
+
 
 def generate_input(rank: int, world_size: int, m: int, n: int, k: int, has_bias: bool, seed: int,
                    device=None) -> input_t:

@@ -35,6 +35,7 @@ from __future__ import annotations
 
 import argparse
 import json
+import math
 import os
 import statistics
 import sys
@@ -441,6 +442,30 @@ def main():
                        "library, what the reference calls) timed the same way beside it",
         }
         del lin, lin_out
+
+        # the whole benchmark list of that task (gemm-rs/task.yml:80-85, ranked by the geometric
+        # mean), each shape timed like the one above, beside the reference's own two statements
+        rows_, ours_, theirs_ = [], [], []
+        for (bm, bn, bk, has_bias, bseed) in gemm_rs.TASK_BENCHMARKS:
+            d = gemm_rs.generate_input(0, 8, bm, bn, bk, has_bias, bseed, device=dev)
+            o = torch.empty(bm, bn, dtype=torch.bfloat16, device=dev)
+
+            def reference_statements():
+                y = torch.matmul(d[0], d[1].T)
+                return y if d[2] is None else y + d[2]
+
+            a_us = timed(lambda: gemm_rs.local_product(d, out=o))
+            r_us = timed(reference_statements)
+            ours_.append(a_us)
+            theirs_.append(r_us)
+            rows_.append({"m": bm, "n": bn, "k_per_rank": bk // 8, "bias": has_bias, "us": round(a_us, 1),
+                          "torch_us": round(r_us, 1)})
+            del d, o
+        geo = lambda v: math.exp(sum(math.log(x) for x in v) / len(v))
+        out["linear"]["task_benchmarks"] = {
+            "shapes": rows_, "geomean_us": round(geo(ours_), 1), "torch_geomean_us": round(geo(theirs_), 1),
+            "note": "per-rank product only (the reduce-scatter between GPUs is not part of either figure)",
+        }
 
     # ---- CPU baseline: the row-by-row torch statement of the same step on the host cores
     if not args.no_cpu:

@@ -349,17 +349,17 @@ int moe_a2a_expert_gemm(const moe_a2a_shape* shape, const void* expert_x,
  * rounded value and the sum rounded again, which is what the two torch
  * statements do. bias may be NULL.
  * One of three kernels runs, picked from the shape alone (so a shape always
- * gives the same bits): from 65 rows on, a kernel bound by the matrix cores,
- * whose workgroups own output tiles of 256 x 256, 128 x 128 or 64 x 128 (the
- * largest that still gives every compute unit work; all three add the same
- * terms in the same order); up to 64 rows, a kernel whose workgroups own 32
- * columns and split k over their waves (partial sums added in a fixed order);
- * otherwise the kernel of moe_a2a_expert_gemm with one group of m rows.
+ * gives the same bits): up to 64 rows and from 512 elements of k, a kernel whose
+ * workgroups own 32 columns and split k over their waves (partial sums added in
+ * a fixed order); else a kernel bound by the matrix cores, whose workgroups own
+ * output tiles of 256 x 256, 128 x 128 or 64 x 128 (the largest that still
+ * gives every compute unit work; all three add the same terms in the same
+ * order); for shapes beyond their index ranges, the kernel of
+ * moe_a2a_expert_gemm with one group of m rows.
  * Limits: n a multiple of 32, k a multiple of 8, input / weight / output 16-byte
  * and bias 8-byte aligned (MOE_A2A_EINVAL / EALIGN). m == 0 is a no-op.
- * The first call on a GPU that takes the first of the three kernels sets kernel
- * attributes (its tiles can use more LDS than a kernel gets by default): make
- * that call outside a graph capture.
+ * The first call on a GPU sets kernel attributes (tiles can use more LDS than a
+ * kernel gets by default): make that call outside a graph capture.
  * The reduce-scatter that follows in the reference (gemm-rs/reference.py:58-59)
  * is an exchange between GPUs and not part of this library.
  */

@@ -16,13 +16,7 @@ from tests.helpers import bits, from_bits
 pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
 
-# (m, n, k of the job, has_bias, seed): gemm-rs/task.yml:56-66 (tests) and :70-75 (benchmarks)
-TASK_TESTS = [(64, 2880, 2880, True, 2035), (64, 3584, 14336, True, 13), (512, 3584, 14336, True, 4297),
-              (512, 4608, 36864, False, 1597), (2048, 4096, 7168, False, 716), (2048, 8192, 30720, False, 20201),
-              (4096, 2880, 2880, True, 136), (4096, 8192, 2048, True, 138), (8192, 3584, 14336, True, 748),
-              (8192, 4608, 36864, True, 4422), (8192, 8192, 28672, False, 1536)]
-TASK_BENCHMARKS = [(64, 7168, 18432, False, 1234), (512, 4096, 12288, True, 663), (2048, 2880, 2880, True, 166),
-                   (4096, 4096, 4096, False, 1371), (8192, 4096, 14336, True, 7168), (8192, 8192, 29568, False, 42)]
+TASK_TESTS, TASK_BENCHMARKS = gemm_rs.TASK_TESTS, gemm_rs.TASK_BENCHMARKS  # gemm-rs/task.yml:66-76, :80-85
 
 
 def check_against_bound(out, inp, weight, bias, name, rows):
@@ -63,10 +57,11 @@ def test_task_shapes(m, n, k, has_bias, seed):
 
 
 @pytest.mark.parametrize("dt", [torch.bfloat16, torch.float16], ids=["bf16", "fp16"])
-# up to 64 rows: with many steps of K a workgroup's waves split K among them, else the grouped kernel
-@pytest.mark.parametrize("m,n,k", [(1, 32, 8), (64, 64, 64), (1, 32, 512), (64, 96, 520), (33, 2880, 1000),
-                                   # from 65 rows: tiles of 64 x 128 (outputs that fill few compute units) ...
-                                   (65, 64, 520), (70, 96, 72), (129, 160, 360), (300, 2880, 200), (70, 64, 1000),
+# up to 64 rows and from 8 steps of K: a workgroup's 4 or 8 waves split K among them, 32 or 64 rows at a time
+@pytest.mark.parametrize("m,n,k", [(1, 32, 512), (64, 96, 520), (33, 2880, 1000), (16, 64, 1600), (64, 96, 1544),
+                                   (32, 32, 3000),
+                                   # else tiles of 64 x 128 (outputs that fill few compute units) ...
+                                   (1, 32, 8), (64, 64, 64), (65, 64, 520), (70, 96, 72), (129, 160, 360), (300, 2880, 200), (70, 64, 1000),
                                    (200, 160, 1096),
                                    # ... of 128 x 128 (short K, or too few tiles of 256 x 256 for every unit) ...
                                    (3000, 2944, 72), (2050, 4128, 200), (4100, 2080, 8), (1000, 4128, 1096),
