@@ -69,6 +69,8 @@ def parse_args():
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="target CPU time of the cpu_baseline sample")
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
     ap.add_argument("--no-gemm", action="store_true", help="skip the grouped GEMM and linear rows")
+    ap.add_argument("--no-gemm-list", action="store_true",
+                    help="skip the list of gemm-rs benchmark shapes inside the linear row (profiles of one shape)")
     ap.add_argument("--no-floor", action="store_true",
                     help="skip the launch-floor measurement (its launches without rows would count into a "
                          "profiler's per-kernel averages)")
@@ -446,7 +448,7 @@ def main():
         # the whole benchmark list of that task (gemm-rs/task.yml:80-85, ranked by the geometric
         # mean), each shape timed like the one above, beside the reference's own two statements
         rows_, ours_, theirs_ = [], [], []
-        for (bm, bn, bk, has_bias, bseed) in gemm_rs.TASK_BENCHMARKS:
+        for (bm, bn, bk, has_bias, bseed) in ([] if args.no_gemm_list else gemm_rs.TASK_BENCHMARKS):
             d = gemm_rs.generate_input(0, 8, bm, bn, bk, has_bias, bseed, device=dev)
             o = torch.empty(bm, bn, dtype=torch.bfloat16, device=dev)
 
@@ -462,10 +464,11 @@ def main():
                           "torch_us": round(r_us, 1)})
             del d, o
         geo = lambda v: math.exp(sum(math.log(x) for x in v) / len(v))
-        out["linear"]["task_benchmarks"] = {
-            "shapes": rows_, "geomean_us": round(geo(ours_), 1), "torch_geomean_us": round(geo(theirs_), 1),
-            "note": "per-rank product only (the reduce-scatter between GPUs is not part of either figure)",
-        }
+        if rows_:
+            out["linear"]["task_benchmarks"] = {
+                "shapes": rows_, "geomean_us": round(geo(ours_), 1), "torch_geomean_us": round(geo(theirs_), 1),
+                "note": "per-rank product only (the reduce-scatter between GPUs is not part of either figure)",
+            }
 
     # ---- CPU baseline: the row-by-row torch statement of the same step on the host cores
     if not args.no_cpu:
