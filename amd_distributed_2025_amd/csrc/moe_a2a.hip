@@ -1719,9 +1719,10 @@ __global__ __launch_bounds__(64 * ROWS) void expert_scale_wave_kernel(
 // (16 rows, same vector) hit all 64 banks once per 16 lanes.
 //
 // The MFMA computes the tile transposed (weights as the A operand, tokens as B), which leaves a lane
-// holding four consecutive output columns of one token: 8-byte stores. Which 8 inputs of a 16-block a
-// lane contributes is the same permutation for both operands, so the sums run over the same
-// products as the textbook order.
+// holding four consecutive output columns of one token: 8-byte stores. MFMA q of a step takes inputs
+// 16 q .. 16 q + 15 of the step (a lane's half kb of them: the 16-byte vector 2 q + kb of the row), the
+// order in which dense_gemm_kernel walks K too: which of the two kernels a row count selects changes no
+// bit of the result.
 //
 // Tiles are numbered over (expert, block of tokens) by a prefix over the device-side counts, so a
 // hot expert is spread over as many workgroups as it has blocks and an empty one costs nothing.
@@ -1813,7 +1814,7 @@ __global__ __launch_bounds__(64 * GW, GW > 4 ? 1 : TJ <= 2 ? MOE_A2A_GEMM_OCC : 
   // Loads are 8 lanes per 128-byte row: lane l of a wave takes row l/8 (+ 8 per further load) and
   // the vector of that row that belongs in physical slot l%8.
   const int sub = lane >> 3, slot = lane & 7;
-  // operand reads: row r of the tile, half kb of the step's inputs, logical vector kb*4 + q
+  // operand reads: row r of the tile, logical vector 2*q + kb of the step (q: the MFMA, kb: the lane's half)
   const int r = lane & 31, kb = lane >> 5, read_swz = (r >> 1) & 7;
 
   const int tiles = row_blocks * col_tiles, stride = gridDim.x;
@@ -1898,13 +1899,13 @@ __global__ __launch_bounds__(64 * GW, GW > 4 ? 1 : TJ <= 2 ? MOE_A2A_GEMM_OCC : 
       for (int i = 0; i < 4; ++i) ws[wave][wslot[i]] = wv[set][i];
       b128 a[4];
 #pragma unroll
-      for (int q = 0; q < 4; ++q) a[q] = ws[wave][r * 8 + ((kb * 4 + q) ^ read_swz)];
+      for (int q = 0; q < 4; ++q) a[q] = ws[wave][r * 8 + ((q * 2 + kb) ^ read_swz)];
 #pragma unroll
       for (int q = 0; q < 4; ++q)
 #pragma unroll
         for (int j = 0; j < TJ; ++j) {
           if (j * 32 < live) {
-            const b128 tok = xs[set][(j * 32 + r) * 8 + ((kb * 4 + q) ^ read_swz)];
+            const b128 tok = xs[set][(j * 32 + r) * 8 + ((q * 2 + kb) ^ read_swz)];
             acc[j] = Mfma32x32x16<DT>::mma(a[q], tok, acc[j]);
           }
         }
@@ -2120,36 +2121,104 @@ __global__ __launch_bounds__(64 * KW) void skinny_gemm_kernel(
 // and consecutive numbers walk GROUP_M tile rows down before they step to the next tile column:
 // the 32 workgroups an XCD runs at a time share 4 row panels of A and 8 of B in its L2.
 
-template <int DT, int WM, int WN, int TM, int TN>
-__global__ __launch_bounds__(64 * WM * WN) void dense_gemm_kernel(
+template <int DT, int WM, int WN, int TM, int TN, bool GROUPED>
+__global__ __launch_bounds__(64 * WM * WN, TM * TN >= 16 ? 1 : 2) void dense_gemm_kernel(
     const b128* __restrict__ A, const b128* __restrict__ B, const uint16_t* __restrict__ bias,
-    uint16_t* __restrict__ C, int M, int N, int K, int tiles_m, int tiles_n) {
+    uint16_t* __restrict__ C, int M, int N, int K, int tiles_m, int tiles_n,
+    const int* __restrict__ rows_of_group, int groups, int max_rows) {
   constexpr int NT = 64 * WM * WN, BM = WM * TM * 32, BN = WN * TN * 32;
   constexpr int LA = BM * 8 / NT, LB = BN * 8 / NT;  // 16-byte vectors a thread copies per step
   constexpr int GROUP_M = 4;
   extern __shared__ b128 tile_lds[];  // [2][(BM + BN) * 8]
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const int wm = __builtin_amdgcn_readfirstlane(wave / WN), wn = __builtin_amdgcn_readfirstlane(wave % WN);
+  const int row_vecs = K / 8, row_bytes = K * 2, steps = (K + GEMM_KSTEP - 1) / GEMM_KSTEP;
+  const int tail_vecs = row_vecs - (steps - 1) * 8;
 
-  int tm, tn;
-  {
+  // GROUPED: A is [groups, max_rows, K], B [groups, N, K], bias [groups, N] or null, C [groups,
+  // max_rows, N], and group g has rows_of_group[g] rows (read here, clamped to max_rows). Row
+  // tiles are numbered over the groups by a prefix over their counts: every thread sums the row
+  // tiles of a run of groups, a scan over the workgroup places the runs, and the thread whose run
+  // holds a row tile walks it to find the group. The launch strides over (row tile, column tile)
+  // pairs, column tile fastest, so its size is a matter of speed only.
+  __shared__ int grp_red[NT / 64];
+  __shared__ int grp_home[2];
+  [[maybe_unused]] auto rows_of = [=](int g) { return min(max(rows_of_group[g], 0), max_rows); };
+  [[maybe_unused]] auto row_tiles_of = [=](int g) { return (rows_of(g) + BM - 1) / BM; };
+  [[maybe_unused]] int run_first = 0, run_begin = 0, run_tiles = 0, total_tiles = 0;
+  if constexpr (GROUPED) {
+    const int per = (groups + NT - 1) / NT;
+    run_first = min(tid * per, groups);
+    const int run_end = min(run_first + per, groups);
+    for (int g = run_first; g < run_end; ++g) run_tiles += row_tiles_of(g);
+    const int inc = wave_inclusive_scan(run_tiles);
+    if (lane == 63) grp_red[wave] = inc;
+    lds_barrier();
+    int off = 0, total = 0;
+#pragma unroll
+    for (int w = 0; w < NT / 64; ++w) {
+      off += w < wave ? grp_red[w] : 0;
+      total += grp_red[w];
+    }
+    run_begin = off + inc - run_tiles;
+    total_tiles = total * tiles_n;
+    if ((int)blockIdx.x >= total_tiles) return;
+  }
+  int tile = blockIdx.x;
+  do {  // (one pass unless GROUPED)
+  int n0, rows_left;          // first column of the tile; rows of A and C from the tile's first row on
+  const b128* a_tile;         // the tile's first row of A
+  const b128* b_tile;         // the tile's first row of B (column n0 of the product)
+  uint16_t* c_tile;           // the tile's first row of C
+  const uint16_t* bias_row;   // the bias of the tile's group, or null
+  if constexpr (GROUPED) {
+    // whole rounds of the launch are renumbered so that an XCD works on consecutive pairs
+    // (the column tiles of one row tile share its rows in that XCD's L2)
+    const int round = tile / (int)gridDim.x;
+    int logical = tile;
+    if ((round + 1) * (int)gridDim.x <= total_tiles)
+      logical = round * (int)gridDim.x + xcd_contiguous(blockIdx.x, gridDim.x);
+    const int rb = logical / tiles_n, tn = logical - rb * tiles_n;
+    lds_barrier();  // the tile before is out of LDS, and its grp_home has been read
+    if (run_begin <= rb && rb < run_begin + run_tiles) {
+      int g = run_first, first = run_begin;
+      for (;; ++g) {
+        const int n = row_tiles_of(g);
+        if (rb < first + n) break;
+        first += n;
+      }
+      grp_home[0] = g;
+      grp_home[1] = first;
+    }
+    lds_barrier();
+    const int g = __builtin_amdgcn_readfirstlane(grp_home[0]);
+    const int t0 = (rb - __builtin_amdgcn_readfirstlane(grp_home[1])) * BM;
+    n0 = tn * BN;
+    rows_left = __builtin_amdgcn_readfirstlane(rows_of(g)) - t0;
+    a_tile = A + ((size_t)g * max_rows + t0) * row_vecs;
+    b_tile = B + ((size_t)g * N + n0) * row_vecs;
+    c_tile = C + ((size_t)g * max_rows + t0) * N;
+    bias_row = bias ? bias + (size_t)g * N : nullptr;
+  } else {
     const int logical = xcd_contiguous(blockIdx.x, gridDim.x);
     const int per_group = GROUP_M * tiles_n, group = logical / per_group, in = logical - group * per_group;
     const int rows = min(GROUP_M, tiles_m - group * GROUP_M);
-    tn = in / rows;
-    tm = group * GROUP_M + in - tn * rows;
+    const int tn = in / rows, tm = group * GROUP_M + in - tn * rows;
+    n0 = tn * BN;
+    rows_left = M - tm * BM;
+    a_tile = A + (size_t)tm * BM * row_vecs;
+    b_tile = B + (size_t)n0 * row_vecs;
+    c_tile = C + (size_t)tm * BM * N;
+    bias_row = bias;
   }
-  const int m0 = tm * BM, n0 = tn * BN;
-  const int row_vecs = K / 8, row_bytes = K * 2, steps = (K + GEMM_KSTEP - 1) / GEMM_KSTEP;
-  const int tail_vecs = row_vecs - (steps - 1) * 8;
 
   // Loads go through buffer descriptors whose extent ends with the last row of the matrix: rows of
   // a tile past it read as zeros. Vectors past the end of a row in the last step are sent out of
   // range the same way.
   const __amdgpu_buffer_rsrc_t abuf = __builtin_amdgcn_make_buffer_rsrc(
-      (void*)(A + (size_t)m0 * row_vecs), 0, min(BM, M - m0) * row_bytes, BUFFER_RAW_32BIT);
+      (void*)a_tile, 0, min(BM, rows_left) * row_bytes, BUFFER_RAW_32BIT);
   const __amdgpu_buffer_rsrc_t bbuf = __builtin_amdgcn_make_buffer_rsrc(
-      (void*)(B + (size_t)n0 * row_vecs), 0, min(BN, N - n0) * row_bytes, BUFFER_RAW_32BIT);
+      (void*)b_tile, 0, min(BN, N - n0) * row_bytes, BUFFER_RAW_32BIT);
   constexpr int OUT_OF_RANGE = 0x40000000;
   // copy i of a thread: LDS place p = tid + i * NT, that is row p / 8 (rows NT / 8 apart, which
   // leaves bits 1..3 of the row number alone) and the vector that belongs in physical slot p % 8
@@ -2161,7 +2230,7 @@ __global__ __launch_bounds__(64 * WM * WN) void dense_gemm_kernel(
   b128 ga[LA], gb[LB];
   // A thread's LA + LB vectors of a step in four quarters: A[0..LA/2), A[LA/2..LA), B[0..LB/2), B[LB/2..LB)
   static_assert(LA % 2 == 0 && LB % 2 == 0, "quarters");
-  auto load_quarter = [&](int q, int step) {
+  auto load_quarter = [&](int q, int step) __attribute__((always_inline)) {
     const int at = min(step, steps - 1);  // (past the end: the last step again, never used)
     const int soff = at * (GEMM_KSTEP * 2), off = coff + (at == steps - 1 ? cpast : 0);
     if (q < 2) {
@@ -2174,7 +2243,7 @@ __global__ __launch_bounds__(64 * WM * WN) void dense_gemm_kernel(
         gb[i] = __builtin_amdgcn_raw_buffer_load_b128(bbuf, off + i * rstep, soff, 0);
     }
   };
-  auto store_quarter = [&](int q, int buf) {
+  auto store_quarter = [&](int q, int buf) __attribute__((always_inline)) {
     b128* as = tile_lds + buf * ((BM + BN) * 8);
     b128* bs = as + BM * 8;
     if (q < 2) {
@@ -2191,7 +2260,7 @@ __global__ __launch_bounds__(64 * WM * WN) void dense_gemm_kernel(
   // Operand fragments of one 16-element slice of a step: two register sets, so that the reads of
   // the next slice are in flight while the matrix cores work on this one.
   b128 af[2][TM], bf[2][TN];
-  auto read_frags = [&](int set, int buf, int kk) {
+  auto read_frags = [&](int set, int buf, int kk) __attribute__((always_inline)) {
     const b128* as = tile_lds + buf * ((BM + BN) * 8) + (wm * TM * 32 + r) * 8;
     const b128* bs = tile_lds + buf * ((BM + BN) * 8) + BM * 8 + (wn * TN * 32 + r) * 8;
     const int v = (kk * 2 + h) ^ swz;
@@ -2200,11 +2269,19 @@ __global__ __launch_bounds__(64 * WM * WN) void dense_gemm_kernel(
 #pragma unroll
     for (int j = 0; j < TN; ++j) bf[set][j] = bs[j * 256 + v];
   };
-  auto mfmas = [&](int set) {
+  // (GROUPED) bands of 32 rows of this wave's part of the tile that hold rows of the group: the
+  // last row tile of a group computes only those, in a copy of the loop with that one condition
+  // (not for the 256 x 256 tile, whose registers have no room for the copy's state: it is used
+  // where groups have many rows, and an empty band is a small part of them)
+  constexpr bool SKIP_BANDS = GROUPED && TM * TN < 16;
+  [[maybe_unused]] const int live_bands = min(max((rows_left - wm * TM * 32 + 31) / 32, 0), TM);
+  auto mfmas = [&](int set, auto ragged) __attribute__((always_inline)) {
 #pragma unroll
-    for (int i = 0; i < TM; ++i)
+    for (int i = 0; i < TM; ++i) {
+      if (decltype(ragged)::value && i >= live_bands) continue;
 #pragma unroll
       for (int j = 0; j < TN; ++j) acc[i][j] = Mfma32x32x16<DT>::mma(bf[set][j], af[set][i], acc[i][j]);
+    }
   };
 
   // Step s computes from LDS buffer s & 1. During it the rows of step s + 1 (in registers since
@@ -2255,35 +2332,40 @@ __global__ __launch_bounds__(64 * WM * WN) void dense_gemm_kernel(
     }                                                                   \
   }                                                                     \
   __builtin_amdgcn_sched_barrier(0);
-  auto one_step = [&](int step, int cur) {  // cur = step & 1, a constant where this is called
+  auto one_step = [&](int step, int cur, auto ragged) __attribute__((always_inline)) {  // cur = step & 1, a constant where this is called
     read_frags(1, cur, 1);
     store_quarter(1, cur ^ 1);
     load_quarter(1, step + 2);
-    mfmas(0);
+    mfmas(0, ragged);
     MOE_A2A_INTERLEAVE()
     read_frags(0, cur, 2);
     store_quarter(2, cur ^ 1);
     load_quarter(2, step + 2);
-    mfmas(1);
+    mfmas(1, ragged);
     MOE_A2A_INTERLEAVE()
     read_frags(1, cur, 3);
     store_quarter(3, cur ^ 1);
     load_quarter(3, step + 2);
-    mfmas(0);
+    mfmas(0, ragged);
     MOE_A2A_INTERLEAVE()
     lds_barrier();
     read_frags(0, cur ^ 1, 0);
     store_quarter(0, cur);
     load_quarter(0, step + 3);
-    mfmas(1);
+    mfmas(1, ragged);
     MOE_A2A_INTERLEAVE()
   };
-  int step = 0;
-  for (; step + 2 <= steps; step += 2) {
-    one_step(step, 0);
-    one_step(step + 1, 1);
-  }
-  if (step < steps) one_step(step, 0);
+  auto walk_k = [&](auto ragged) __attribute__((always_inline)) {
+    int step = 0;
+    for (; step + 2 <= steps; step += 2) {
+      one_step(step, 0, ragged);
+      one_step(step + 1, 1, ragged);
+    }
+    if (step < steps) one_step(step, 0, ragged);
+  };
+  // (both copies hold the same barriers, so the waves of a workgroup may take different ones)
+  if (!SKIP_BANDS || live_bands == TM) walk_k(std::false_type{});
+  else if constexpr (SKIP_BANDS) walk_k(std::true_type{});
 
   // Results leave through LDS so that they reach memory in whole lines. acc[i][j] holds row
   // i*32 + r of the wave's tile and columns j*32 + g*8 + h*4 + 0..3 (g < 4): a lane's own values
@@ -2299,16 +2381,17 @@ __global__ __launch_bounds__(64 * WM * WN) void dense_gemm_kernel(
     char* park = (char*)tile_lds + wave * (32 * PITCH);
     const int ncol = n0 + wn * TN * 32;
     uint32_t bias2[TN][4][2] = {};
-    if (bias) {
+    if (bias_row) {
 #pragma unroll
       for (int j = 0; j < TN; ++j)
 #pragma unroll
         for (int g = 0; g < 4; ++g)
-          if (ncol + j * 32 < N) __builtin_memcpy(bias2[j][g], bias + ncol + j * 32 + g * 8 + h * 4, 8);
+          if (ncol + j * 32 < N) __builtin_memcpy(bias2[j][g], bias_row + ncol + j * 32 + g * 8 + h * 4, 8);
     }
     const int rrow = lane / VR, rvec = lane % VR;
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
+      if (SKIP_BANDS && i >= live_bands) continue;
 #pragma unroll
       for (int j = 0; j < TN; ++j) {
         const f32x16& c = acc[i][j];
@@ -2316,7 +2399,7 @@ __global__ __launch_bounds__(64 * WM * WN) void dense_gemm_kernel(
         for (int g = 0; g < 4; ++g) {
           uint32_t two[2] = {Pair16<DT>::canonical(Pair16<DT>::round(c[g * 4 + 0], c[g * 4 + 1])),
                              Pair16<DT>::canonical(Pair16<DT>::round(c[g * 4 + 2], c[g * 4 + 3]))};
-          if (bias) {
+          if (bias_row) {
 #pragma unroll
             for (int e = 0; e < 2; ++e)
               two[e] = Pair16<DT>::canonical(Pair16<DT>::round(
@@ -2330,11 +2413,13 @@ __global__ __launch_bounds__(64 * WM * WN) void dense_gemm_kernel(
       for (int p = 0; p < 32 / ROWS_PER_READ; ++p) {
         const int row = p * ROWS_PER_READ + rrow;
         const b128 v = *(const b128*)(park + row * PITCH + rvec * 16);
-        const int m = m0 + (wm * TM + i) * 32 + row, n = ncol + rvec * 8;
-        if (m < M && n < N) *(b128*)(C + (size_t)m * N + n) = v;
+        const int m = (wm * TM + i) * 32 + row, n = ncol + rvec * 8;
+        if (m < rows_left && n < N) *(b128*)(c_tile + (size_t)m * N + n) = v;
       }
     }
   }
+  tile += gridDim.x;
+  } while (GROUPED && tile < total_tiles);
 }
 
 #undef MOE_A2A_INTERLEAVE
@@ -3028,12 +3113,18 @@ int allow_large_lds() {
   auto allow = [&](const void* kernel, size_t bytes) {
     ok = ok && hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes) == hipSuccess;
   };
-  allow((const void*)dense_gemm_kernel<MOE_A2A_BF16, 2, 2, 4, 4>, dense_lds_bytes(256, 256));
-  allow((const void*)dense_gemm_kernel<MOE_A2A_F16, 2, 2, 4, 4>, dense_lds_bytes(256, 256));
-  allow((const void*)dense_gemm_kernel<MOE_A2A_BF16, 2, 2, 2, 2>, dense_lds_bytes(128, 128));
-  allow((const void*)dense_gemm_kernel<MOE_A2A_F16, 2, 2, 2, 2>, dense_lds_bytes(128, 128));
-  allow((const void*)dense_gemm_kernel<MOE_A2A_BF16, 2, 2, 1, 2>, dense_lds_bytes(64, 128));
-  allow((const void*)dense_gemm_kernel<MOE_A2A_F16, 2, 2, 1, 2>, dense_lds_bytes(64, 128));
+  allow((const void*)dense_gemm_kernel<MOE_A2A_BF16, 2, 2, 4, 4, false>, dense_lds_bytes(256, 256));
+  allow((const void*)dense_gemm_kernel<MOE_A2A_F16, 2, 2, 4, 4, false>, dense_lds_bytes(256, 256));
+  allow((const void*)dense_gemm_kernel<MOE_A2A_BF16, 2, 2, 2, 2, false>, dense_lds_bytes(128, 128));
+  allow((const void*)dense_gemm_kernel<MOE_A2A_F16, 2, 2, 2, 2, false>, dense_lds_bytes(128, 128));
+  allow((const void*)dense_gemm_kernel<MOE_A2A_BF16, 2, 2, 1, 2, false>, dense_lds_bytes(64, 128));
+  allow((const void*)dense_gemm_kernel<MOE_A2A_F16, 2, 2, 1, 2, false>, dense_lds_bytes(64, 128));
+  allow((const void*)dense_gemm_kernel<MOE_A2A_BF16, 2, 2, 4, 4, true>, dense_lds_bytes(256, 256));
+  allow((const void*)dense_gemm_kernel<MOE_A2A_F16, 2, 2, 4, 4, true>, dense_lds_bytes(256, 256));
+  allow((const void*)dense_gemm_kernel<MOE_A2A_BF16, 2, 2, 2, 2, true>, dense_lds_bytes(128, 128));
+  allow((const void*)dense_gemm_kernel<MOE_A2A_F16, 2, 2, 2, 2, true>, dense_lds_bytes(128, 128));
+  allow((const void*)dense_gemm_kernel<MOE_A2A_BF16, 2, 2, 1, 2, true>, dense_lds_bytes(64, 128));
+  allow((const void*)dense_gemm_kernel<MOE_A2A_F16, 2, 2, 1, 2, true>, dense_lds_bytes(64, 128));
   allow((const void*)skinny_gemm_kernel<MOE_A2A_BF16, 2, 8>, skinny_lds_bytes(2, 8));
   allow((const void*)skinny_gemm_kernel<MOE_A2A_F16, 2, 8>, skinny_lds_bytes(2, 8));
   if (!ok) return MOE_A2A_ELAUNCH;
@@ -3057,8 +3148,9 @@ int launch_dense_gemm(const void* a, const void* b, const void* bias, void* c, i
   const int grid = (int)(tiles_m * tiles_n);
   if (const int rc = allow_large_lds()) return rc;
 #define LAUNCH_D(DT, TM, TN)                                                             \
-  dense_gemm_kernel<DT, 2, 2, TM, TN><<<grid, 256, lds_bytes, st>>>(                     \
-      (const b128*)a, (const b128*)b, (const uint16_t*)bias, (uint16_t*)c, M, N, K, (int)tiles_m, (int)tiles_n)
+  dense_gemm_kernel<DT, 2, 2, TM, TN, false><<<grid, 256, lds_bytes, st>>>(              \
+      (const b128*)a, (const b128*)b, (const uint16_t*)bias, (uint16_t*)c, M, N, K, (int)tiles_m, (int)tiles_n, \
+      nullptr, 0, 0)
 #define LAUNCH_DT(DT)                         \
   do {                                        \
     if (tile == 256) LAUNCH_D(DT, 4, 4);      \
@@ -3069,6 +3161,57 @@ int launch_dense_gemm(const void* a, const void* b, const void* bias, void* c, i
   else LAUNCH_DT(MOE_A2A_F16);
 #undef LAUNCH_DT
 #undef LAUNCH_D
+  return launch_status();
+}
+
+#ifndef MOE_A2A_GROUPED_DENSE_MIN_ROWS
+#define MOE_A2A_GROUPED_DENSE_MIN_ROWS 56  // rows per group (from the caller's row count) from which tiles are used
+#endif
+#ifndef MOE_A2A_GROUPED_DENSE_BIG_ROWS
+#define MOE_A2A_GROUPED_DENSE_BIG_ROWS 768  // ... and from which they are 256 x 256 instead of 128 x 128
+#endif
+
+// The grouped product when groups have hundreds of rows: the weights are then read for enough
+// rows that the matrix cores, not the stream of weights, bound the work, and the dense kernel's
+// tiles (each weight row read once per 128 or 256 rows, operands shared by four waves through
+// LDS) do better than the kernel that is built around streaming. MOE_A2A_NOT_DENSE otherwise.
+int launch_grouped_dense(const void* x, const int32_t* rows_of_group, const void* w, void* y, int groups,
+                         long long max_rows, long long rows_hint, int N, int K, int dtype, hipStream_t st) {
+  if (dtype != MOE_A2A_F16 && dtype != MOE_A2A_BF16) return MOE_A2A_EINVAL;
+  if (N % 32 != 0 || K % 8 != 0) return MOE_A2A_EINVAL;
+  if (!all_aligned(16, x, w, y)) return MOE_A2A_EALIGN;
+  if (!rows_of_group || rows_hint < (long long)MOE_A2A_GROUPED_DENSE_MIN_ROWS * groups) return MOE_A2A_NOT_DENSE;
+  if ((long long)K * 2 * 256 >= (1 << 30) || max_rows > INT_MAX / 2) return MOE_A2A_NOT_DENSE;
+#ifndef MOE_A2A_GROUPED_DENSE_TILE
+#define MOE_A2A_GROUPED_DENSE_TILE 0  // (measurements) 256, 128 or 64: that tile height for every launch
+#endif
+  // 256 x 256 when groups have rows for several bands of them; 64 x 128 when tiles of 128 x 128
+  // would not give every compute unit one
+  const int tile = MOE_A2A_GROUPED_DENSE_TILE ? MOE_A2A_GROUPED_DENSE_TILE
+                   : rows_hint >= (long long)MOE_A2A_GROUPED_DENSE_BIG_ROWS * groups ? 256
+                   : (rows_hint / 128 + groups) * ((N + 127) / 128) <= 256 ? 64 : 128;
+  const int BM = tile, BN = tile == 64 ? 128 : tile;
+  const long long tiles_n = (N + BN - 1) / BN;
+  // every group can end in a partly filled row tile; the kernel strides over what the hint misses
+  const long long pairs = (rows_hint / BM + groups) * tiles_n;
+  if ((max_rows / BM + 1) * groups * tiles_n > INT_MAX / 2) return MOE_A2A_NOT_DENSE;
+  const int grid = mover_blocks(pairs);
+  const size_t lds_bytes = dense_lds_bytes(BM, BN);
+  if (const int rc = allow_large_lds()) return rc;
+#define LAUNCH_GD(DT, TM, TN)                                                                 \
+  dense_gemm_kernel<DT, 2, 2, TM, TN, true><<<grid, 256, lds_bytes, st>>>(                    \
+      (const b128*)x, (const b128*)w, nullptr, (uint16_t*)y, 0, N, K, 0, (int)tiles_n, rows_of_group, groups, \
+      (int)max_rows)
+  if (dtype == MOE_A2A_BF16) {
+    if (tile == 256) LAUNCH_GD(MOE_A2A_BF16, 4, 4);
+    else if (tile == 128) LAUNCH_GD(MOE_A2A_BF16, 2, 2);
+    else LAUNCH_GD(MOE_A2A_BF16, 1, 2);
+  } else {
+    if (tile == 256) LAUNCH_GD(MOE_A2A_F16, 4, 4);
+    else if (tile == 128) LAUNCH_GD(MOE_A2A_F16, 2, 2);
+    else LAUNCH_GD(MOE_A2A_F16, 1, 2);
+  }
+#undef LAUNCH_GD
   return launch_status();
 }
 
@@ -3125,6 +3268,9 @@ int moe_a2a_expert_gemm(const moe_a2a_shape* s, const void* expert_x,
     return MOE_A2A_EINVAL;
   const int nle = s->num_experts / s->world_size;
   const long long max_recv = (long long)s->max_num_tokens * s->world_size;
+  const int dense = launch_grouped_dense(expert_x, expert_num_tokens, weights, expert_y, nle, max_recv, rows_hint,
+                                         s->hidden_dim, s->hidden_dim, dtype, (hipStream_t)stream);
+  if (dense != MOE_A2A_NOT_DENSE) return dense;
   return launch_grouped_gemm(expert_x, expert_num_tokens, weights, nullptr, expert_y, nle, max_recv,
                              rows_hint, s->hidden_dim, s->hidden_dim, dtype, (hipStream_t)stream);
 }

@@ -323,10 +323,16 @@ int moe_a2a_expert_scale(const moe_a2a_shape* shape, const void* expert_x,
  *   dtype      MOE_A2A_F16 or MOE_A2A_BF16: element type of all three
  *   expert_y   [nle, max_recv, H] out; rows at or past expert_num_tokens[le] are
  *              not written
- * Rows are processed in blocks of 64 or 128 tokens found from the device-side
- * counts, so the work follows the rows, not the experts; with blocks of 128
- * tokens a workgroup is 160 to 256 columns wide, the width picked from
- * rows_hint so that the launch fills the compute units in whole rounds. Limits: hidden_dim a
+ * Rows are processed in blocks found from the device-side counts, so the work
+ * follows the rows, not the experts. rows_hint (the rows the caller expects
+ * over all experts) picks the kernel and sizes the launch, and changes no bit
+ * of the result: from about 56 rows per expert, output tiles of 128 x 128
+ * (64 x 128 when those would be too few for the GPU, 256 x 256 from about 768
+ * rows per expert) of the kernel behind moe_a2a_linear, numbered over the
+ * experts; below, a kernel built around streaming every weight once, in blocks
+ * of 64 or 128 tokens and workgroups 128 to 256 columns wide. The first call on
+ * a GPU sets kernel attributes (tiles can use more LDS than a kernel gets by
+ * default): make that call outside a graph capture. Limits: hidden_dim a
  * multiple of 32, all three buffers 16-byte aligned (MOE_A2A_EINVAL / EALIGN).
  * Sums are formed in float32 in the order of the matrix unit, which is not the
  * order of a CPU matmul: results lie within what float32 accumulation in any

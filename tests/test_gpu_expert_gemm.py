@@ -224,3 +224,26 @@ def test_wide_workgroups_of_every_width(H, width):
         zero = (want & 0x7FFF) == 0
         assert np.array_equal(got[le, :c][~zero], want[~zero]), f"expert {le}"
         assert ((got[le, :c][zero] & 0x7FFF) == 0).all()
+
+
+@pytest.mark.parametrize("dt", [torch.bfloat16, torch.float16], ids=["bf16", "fp16"])
+@pytest.mark.parametrize("nle,H,max_tokens,counts", [
+    # about 160 rows per expert and more: tiles of 128 x 128 (ragged last tiles in both directions, an empty
+    # expert, exact multiples of the tile, one row)
+    (6, 416, 400, [384, 0, 5, 400, 131, 256]),
+    (5, 7168, 300, [290, 213, 0, 256, 129]),
+    # about 768 rows and more: tiles of 256 x 256
+    (3, 320, 1100, [1100, 770, 513]),
+    (2, 1024, 1030, [1025, 1024]),
+])
+def test_tiles_for_experts_with_hundreds_of_rows(nle, H, max_tokens, counts, dt):
+    """From about 160 rows per expert (judged from the row count the caller passes) the product runs on the
+    dense kernel's tiles, found over the experts from the device-side counts. The row count only picks the
+    kernel and sizes the launch: every value of it gives the same bits, those of the streaming kernel
+    (hint 0) included, within the float32 bound, and rows past the counts stay untouched."""
+    print(f"gemm tiles nle={nle} H={H} counts={counts} {dt}", flush=True)
+    a, cfg = rank_object(1, nle, H, max_tokens, dt)
+    total = sum(counts)
+    full = random_case(a, cfg, 1, counts, seed=21, hint=total, check_experts=[0, nle - 1] if H > 2048 else None)
+    for hint in (0, 160 * nle, 768 * nle, 10 * total):
+        assert np.array_equal(run_gemm_same(a, cfg, 1, counts, 21, hint), full), f"hint {hint}"
