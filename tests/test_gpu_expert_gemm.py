@@ -194,20 +194,22 @@ def test_unsupported_shapes_raise():
 
 @pytest.mark.parametrize("H,width", [(576, 5), (640, 6), (704, 7), (832, 8)])
 def test_wide_workgroups_of_every_width(H, width):
-    """With blocks of 128 tokens and many tiles a workgroup is 5 to 8 waves wide, the width picked
-    from the row count so that the launch fills the compute units in whole rounds: 128 experts of
-    about 60 rows and these four row lengths take the four widths (5 to 7 waves leave the token
-    loads to the first four). Signed permutation weights: exact."""
+    """The streaming kernel between 48 and 56 rows per expert (above, the product runs on tiles): with
+    blocks of 128 tokens and many tiles a workgroup is 5 to 8 waves wide, the width picked from the row
+    count so that the launch fills the compute units in whole rounds: 128 experts of about 52 rows and
+    these four row lengths take the four widths (5 to 7 waves leave the token loads to the first four).
+    Signed permutation weights: exact."""
     print(f"wide workgroups: H={H}, expected width {width} waves", flush=True)
     dt, nle, max_tokens = torch.bfloat16, 128, 140
     rng = np.random.default_rng(H)
     a, cfg = rank_object(1, nle, H, max_tokens, dt)
-    counts = [60] * nle
-    for i, c in enumerate([0, 140, 1, 129, 128, 127, 33]):   # ragged, and the total stays 60 * nle
-        counts[i], counts[nle - 1 - i] = c, 120 - c if c <= 120 else 0
+    counts = [52] * nle
+    for i, c in enumerate([0, 1, 129, 128, 127, 33]):   # ragged, and the total stays 52 * nle
+        counts[2 + i], counts[nle - 3 - i] = c, 104 - c if c <= 104 else 0
     counts[1], counts[nle - 2] = 140, 0
-    total = 60 * nle
-    counts[nle // 2] += total - sum(counts)
+    total = 52 * nle
+    for i in range(20, 20 + (sum(counts) - total) // 2):
+        counts[i] -= 2
     assert sum(counts) == total and 0 <= min(counts) and max(counts) <= max_tokens
     xb = rng.integers(0, 1 << 16, (nle, max_tokens, H), dtype=np.uint16)
     xb[~np.isfinite(orc.b16_to_f32(xb, "bf16"))] = 0x3C00
