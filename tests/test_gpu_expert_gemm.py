@@ -249,3 +249,47 @@ def test_tiles_for_experts_with_hundreds_of_rows(nle, H, max_tokens, counts, dt)
     full = random_case(a, cfg, 1, counts, seed=21, hint=total, check_experts=[0, nle - 1] if H > 2048 else None)
     for hint in (0, 160 * nle, 768 * nle, 10 * total):
         assert np.array_equal(run_gemm_same(a, cfg, 1, counts, 21, hint), full), f"hint {hint}"
+
+
+def test_graph_replays_of_both_products_match_eager():
+    """The grouped product (on tiles, and the streaming kernel through a low row count) and the gemm-rs
+    product captured in a HIP graph after one warm-up call each (the first call on a GPU sets kernel
+    attributes): every replay, with new operands and eager work in between, gives the eager bits."""
+    from amd_distributed_2025_amd import gemm_rs
+    dt, nle, H, T = torch.bfloat16, 6, 512, 300
+    a, cfg = rank_object(1, nle, H, T, dt)
+    counts = [300, 0, 131, 64, 257, 5]
+    num = torch.tensor(counts, dtype=torch.int32, device=DEV)
+    g = torch.Generator(device=DEV).manual_seed(4)
+    ex = torch.randn(nle, T, H, generator=g, device=DEV).to(dt)
+    w = (torch.randn(nle, H, H, generator=g, device=DEV) / H ** 0.5).to(dt)
+    lin = gemm_rs.generate_input(0, 8, 512, 4096, 12288, True, 663, device=DEV)
+    lin_out = torch.empty(512, 4096, dtype=dt, device=DEV)
+    outs = {}
+
+    def step():
+        outs["tiles"] = a.expert_gemm(ex, num, w, sum(counts))
+        outs["linear"] = gemm_rs.local_product(lin, out=lin_out)
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        step()                                   # warm-up outside the capture
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        step()
+    for i in range(3):
+        ex.copy_(torch.randn(nle, T, H, generator=g, device=DEV).to(dt))   # new operands, eager work between replays
+        lin[0].mul_(-1.0)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        got_tiles, got_lin = outs["tiles"].clone(), outs["linear"].clone()
+        want_tiles = a.expert_gemm(ex, num, w, 0).clone()   # eager, the streaming kernel: the same bits
+        want_lin = gemm_rs.local_product(lin).clone()
+        torch.cuda.synchronize()
+        for le, c in enumerate(counts):
+            assert torch.equal(got_tiles[le, :c], want_tiles[le, :c]), f"replay {i}, expert {le}"
+        assert torch.equal(got_lin, want_lin), f"replay {i}: linear"
