@@ -13,7 +13,7 @@ one rank (where the reduce-scatter is the identity) and refuses larger ones.
 """
 from __future__ import annotations
 
-from typing import Optional, Tuple
+from typing import List, Optional, Sequence, Tuple
 
 import torch
 
@@ -81,3 +81,28 @@ def custom_kernel(data: input_t) -> torch.Tensor:
         raise NotImplementedError("the reduce-scatter over several GPUs is outside this package; "
                                   "local_product() gives this rank's [M, N] partial product")
     return local_product(data)
+
+
+def reduce_scatter_local(partials: Sequence[torch.Tensor], rank: int) -> torch.Tensor:
+    """Stand-in, on one GPU, for the `reduce_scatter_tensor` that ends the reference's kernel
+    (gemm-rs/reference.py:58-59): rank `rank`'s [M / W, N] slice of the sum of all W ranks'
+    [M, N] partial products. The sum is formed in float32 in rank order and rounded once; the
+    collective's own order and intermediate roundings are the library's, so results agree with
+    it within the task's tolerance (rtol = atol = 1e-2, reference.py:66), not to the bit."""
+    world_size = len(partials)
+    m, n = partials[0].shape
+    if m % world_size:
+        raise ValueError("m must be divisible by world_size")
+    rows = slice(rank * (m // world_size), (rank + 1) * (m // world_size))
+    total = partials[0][rows].float()
+    for p in partials[1:]:
+        total += p[rows].float()
+    return total.to(partials[0].dtype)
+
+
+def run_job(world: Sequence[input_t], binding: str = "ctypes") -> List[torch.Tensor]:
+    """All ranks of a job on one GPU: every rank's local product through `moe_a2a_linear`, then
+    the stand-in reduce-scatter. Returns the ranks' [M / W, N] outputs. (As in the reference,
+    every rank adds the bias before the sum, so the result holds it W times.)"""
+    partials = [local_product(data, binding=binding) for data in world]
+    return [reduce_scatter_local(partials, r) for r in range(len(world))]

@@ -126,3 +126,37 @@ def test_arguments_are_checked():
     with pytest.raises(ValueError):
         gemm_rs.local_product((x.cpu(), w.cpu(), None))
     assert gemm_rs.custom_kernel((x, w, None)).shape == (4, 32)
+
+
+@pytest.mark.parametrize("m,n,k,has_bias,seed", [(64, 2880, 2880, True, 2035), (512, 4608, 36864, False, 1597),
+                                                 (2048, 4096, 7168, False, 716), (4096, 2880, 2880, True, 136)])
+def test_ranks_of_a_job_sum_to_the_whole_product(m, n, k, has_bias, seed):
+    """The task as a whole on one GPU: the 8 ranks' local products over their slices of K, summed by the
+    stand-in reduce-scatter, against the float64 product over all of K plus 8 times the bias (every rank
+    adds it before the sum, gemm-rs/reference.py:55-59), at the task's tolerance (reference.py:66) and at
+    the bound the roundings to bf16 allow."""
+    W = 8
+    world = [gemm_rs.generate_input(r, W, m, n, k, has_bias, seed, device=DEV) for r in range(W)]
+    outs = gemm_rs.run_job(world)
+    whole = torch.zeros(m, n, dtype=torch.float64, device=DEV)
+    size = torch.zeros(m, n, dtype=torch.float64, device=DEV)   # sum of the magnitudes that get rounded
+    for inp, weight, bias in world:
+        part = inp.double() @ weight.double().T
+        if bias is not None:
+            size += part.abs()
+            part = part + bias.double()
+        whole += part
+        size += part.abs()
+    size += whole.abs()
+    for r, out in enumerate(outs):
+        assert out.shape == (m // W, n) and out.dtype == torch.bfloat16
+        rows = slice(r * (m // W), (r + 1) * (m // W))
+        assert torch.allclose(out.double(), whole[rows], rtol=1e-2, atol=1e-2), f"rank {r}"
+        # and far inside it: every value that is rounded to bf16 on the way (each rank's product, its sum
+        # with the bias, the total) may be off by 2^-9 of its size; float32 sums add far less
+        err = (out.double() - whole[rows]).abs()
+        assert (err <= 2.0 ** -8 * size[rows] + 1e-9).all(), f"rank {r}: {float(err.max()):.3e}"
+    # the ranks share the bias (drawn from the job's seed) and differ in their operands
+    if has_bias:
+        assert torch.equal(world[0][2], world[W - 1][2])
+    assert not torch.equal(world[0][0], world[1][0])
