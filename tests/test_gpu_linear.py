@@ -160,3 +160,39 @@ def test_ranks_of_a_job_sum_to_the_whole_product(m, n, k, has_bias, seed):
     if has_bias:
         assert torch.equal(world[0][2], world[W - 1][2])
     assert not torch.equal(world[0][0], world[1][0])
+
+
+def _random_shapes(seed):
+    rng = np.random.default_rng(seed)
+    shapes = []
+    for lo_m, hi_m, hi_n, count in ((1, 65, 70, 12), (65, 1400, 70, 10), (1500, 4200, 140, 10)):
+        for _ in range(count):
+            k = 8 * int(rng.choice([rng.integers(1, 9), rng.integers(9, 64), rng.integers(64, 200)]))
+            shapes.append((int(rng.integers(lo_m, hi_m)), 32 * int(rng.integers(hi_n // 2, hi_n)), k))
+    return shapes
+
+
+@pytest.mark.parametrize("m,n,k", _random_shapes(20251))
+def test_random_shapes_of_small_integers_are_exact(m, n, k):
+    """Shapes drawn at random across the ranges that pick each kernel and tile (few rows with K split over
+    waves, tiles of 64 x 128, 128 x 128 and 256 x 256), ragged in every direction: small integers with a
+    bias must come out exactly, with stray NaNs around the operands and sentinels around the result."""
+    print(f"linear random shape m={m} n={n} k={k}", flush=True)
+    dt = torch.bfloat16
+    rng = np.random.default_rng(m * 7919 + n * 31 + k)
+    x = rng.integers(-1, 2, (m, k))
+    w = rng.integers(-1, 2, (n, k))
+    b = rng.integers(-8, 9, n)
+    pad = torch.full((m + 2, k), float("nan"), dtype=dt, device=DEV)
+    pad[1:m + 1] = torch.from_numpy(x).to(dt)
+    wpad = torch.full((n + 2, k), float("nan"), dtype=dt, device=DEV)
+    wpad[1:n + 1] = torch.from_numpy(w).to(dt)
+    bias = torch.from_numpy(b).to(dt).to(DEV)
+    out = torch.full((m + 2, n), 777.0, dtype=dt, device=DEV)
+    gemm_rs.local_product((pad[1:m + 1], wpad[1:n + 1], bias), out=out[1:m + 1])
+    torch.cuda.synchronize()
+    prod = (x.astype(np.float64) @ w.T.astype(np.float64)).astype(np.int64)
+    want = prod + b[None, :]
+    assert np.abs(want).max() <= 256 and np.abs(prod).max() <= 256
+    assert np.array_equal(out[1:m + 1].float().cpu().numpy(), want.astype(np.float32))
+    assert (out[0] == 777.0).all() and (out[m + 1] == 777.0).all()
