@@ -293,3 +293,29 @@ def test_graph_replays_of_both_products_match_eager():
         for le, c in enumerate(counts):
             assert torch.equal(got_tiles[le, :c], want_tiles[le, :c]), f"replay {i}, expert {le}"
         assert torch.equal(got_lin, want_lin), f"replay {i}: linear"
+
+
+def _random_layouts(seed, count):
+    rng = np.random.default_rng(seed)
+    cases = []
+    for _ in range(count):
+        nle = int(rng.integers(1, 41))
+        H = 32 * int(rng.integers(1, 30))
+        max_tokens = int(rng.choice([40, 130, 300, 600]))
+        counts = [int(c) for c in rng.integers(0, max_tokens + 1, nle)]
+        for i, c in enumerate(rng.choice([0, 1, 31, 32, 33, 64, 127, 128, 129, 256, 257, max_tokens], 3)):
+            counts[int(rng.integers(0, nle))] = min(int(c), max_tokens)
+        cases.append((nle, H, max_tokens, counts))
+    return cases
+
+
+@pytest.mark.parametrize("nle,H,max_tokens,counts", _random_layouts(77, 14))
+def test_random_layouts_give_the_same_bits_on_every_kernel(nle, H, max_tokens, counts):
+    """Random numbers of experts, row lengths and ragged counts: the streaming kernel (row count 0), tiles of
+    64 x 128 or 128 x 128 (a row count of 56 per expert or the true one) and tiles of 256 x 256 (768 per
+    expert) give the same bits, inside the float32 bound, and leave the rows past the counts alone."""
+    print(f"gemm random layout nle={nle} H={H} T={max_tokens} rows={sum(counts)}", flush=True)
+    a, cfg = rank_object(1, nle, H, max_tokens, torch.bfloat16)
+    base = random_case(a, cfg, 1, counts, seed=nle * 1000 + H, hint=0, check_experts=[0, nle - 1])
+    for hint in (max(sum(counts), 56 * nle), 768 * nle):
+        assert np.array_equal(run_gemm_same(a, cfg, 1, counts, nle * 1000 + H, hint), base), f"hint {hint}"
