@@ -306,6 +306,10 @@ def _random_layouts(seed, count):
         for i, c in enumerate(rng.choice([0, 1, 31, 32, 33, 64, 127, 128, 129, 256, 257, max_tokens], 3)):
             counts[int(rng.integers(0, nle))] = min(int(c), max_tokens)
         cases.append((nle, H, max_tokens, counts))
+    # more experts than a workgroup has threads: every thread sums the row tiles of a run of experts
+    many = [int(c) for c in rng.integers(0, 131, 600)]
+    many[0], many[299], many[599] = 130, 0, 129
+    cases.append((600, 64, 130, many))
     return cases
 
 
