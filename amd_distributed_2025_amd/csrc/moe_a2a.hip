@@ -84,8 +84,8 @@ __device__ __forceinline__ void row_store(V* p, const V& v) {
   if constexpr (NT) __builtin_nontemporal_store(v, p);
   else *p = v;
 }
-template <typename V>
-__device__ __forceinline__ V stream_load(const V* p) {
+template <typename P>
+__device__ __forceinline__ auto stream_load(P p) {
 #if MOE_A2A_NT_LOAD
   return __builtin_nontemporal_load(p);
 #else
@@ -144,6 +144,32 @@ __device__ __forceinline__ int block_sum(int v, int* red) {
   lds_barrier();
   return s;
 }
+
+// A value that was loaded early, handed on at the place where the program first needs it. The
+// compiler moves arithmetic on a loaded value (a clamp, a compare) up to the load, out of loops
+// and branches, and then waits for the load right there: a whole memory round trip ahead of
+// everything issued after it. An empty volatile asm statement cannot be moved, so the wait lands
+// where this is called.
+__device__ __forceinline__ int first_use(int v) {
+  asm volatile("" : "+v"(v));
+  return v;
+}
+
+// Loads through a pointer that went through unknown_origin() and were issued before issued_here()
+// stay before it. The compiler otherwise sinks a load whose value is only used under a condition
+// into that condition's block, behind whatever the condition waits for; an asm statement that
+// may write memory stops that only for pointers that it cannot prove untouched by the statement
+// (a __restrict__ parameter is proven, the same address out of an asm statement is not).
+// The pointer must be the same for every lane of the wave (it is kept in scalar registers).
+template <typename T>
+using global_ptr = const T __attribute__((address_space(1)))*;  // (still known to point into global memory)
+template <typename T>
+__device__ __forceinline__ global_ptr<T> unknown_origin(const T* p) {
+  uint64_t a = (uint64_t)p;
+  asm volatile("" : "+s"(a));
+  return (global_ptr<T>)a;
+}
+__device__ __forceinline__ void issued_here() { asm volatile("" ::: "memory"); }
 
 // Workgroups are handed to the 8 XCDs round-robin by blockIdx. This bijection
 // on [0, grid) gives each XCD one contiguous run of logical items, so items
@@ -264,7 +290,8 @@ struct StridedKeys {
 template <typename V, int NVW>
 struct WavePayload {
   V v[NVW];
-  __device__ __forceinline__ void load(const V* __restrict__ row, int base, int row_vecs, int lane) {
+  template <typename P>  // const V* or global_ptr<V>
+  __device__ __forceinline__ void load(P row, int base, int row_vecs, int lane) {
 #pragma unroll
     for (int j = 0; j < NVW; ++j) v[j] = stream_load(row + min(base + j * 64 + lane, row_vecs - 1));
   }
@@ -432,7 +459,17 @@ __global__ __launch_bounds__(64 * ROWS) void dispatch_send_kernel(
 // [0, E): entry a precedes entry b exactly when its composite key is smaller.
 // The host uses this kernel when (W + 2) * S fits an int.
 
-constexpr int FAN = 8;
+// Entries of a token that are ranked in one pass over the keys and then stored (2, 4 or 8). Fewer
+// per pass means more passes over the same keys (they stay in registers) and more barriers, but the
+// first rows leave sooner and the ranking of the next entries runs while they drain; a compute
+// unit has nothing else to do meanwhile, because all its workgroups rank at the same time.
+// Measured at K = 8, H = 7168: the four path kernels together take 0.5 us less with 4 than with 8
+// and another 0.1 to 0.3 us less with 2.
+#ifndef MOE_A2A_FAN
+#define MOE_A2A_FAN 2
+#endif
+constexpr int FAN = MOE_A2A_FAN;
+static_assert(FAN == 2 || FAN == 4 || FAN == 8, "pairs of 16-bit counts, at most one DPP row of 16 lanes per pair");
 
 template <typename V, int NV>
 __global__ __launch_bounds__(BLOCK) void dispatch_fanout_kernel(
@@ -575,6 +612,10 @@ __global__ __launch_bounds__(BLK) void dispatch_fanout_wide_kernel(
     const int col = c * (BLK * NV) + tid;  // this lane's first vector; the others BLK apart
     const int i0 = t * K;
 
+    // the token's own expert ids, FAN at a time: lane l of every wave holds entry g0 + l % FAN. One
+    // vector load issued ahead of the keys (as uniform loads they become scalar loads that are
+    // waited for one by one in the middle of the ranking)
+    const int own0 = indices[i0 + min(lane & (FAN - 1), K - 1)];
     int key[KEYS];
 #pragma unroll
     for (int u = 0; u < KEYS; ++u) key[u] = indices[min(tid + u * BLK, S - 1)];
@@ -583,11 +624,15 @@ __global__ __launch_bounds__(BLK) void dispatch_fanout_wide_kernel(
     for (int j = 0; j < NV; ++j) v[j] = stream_load(x + (size_t)t * row_vecs + min(col + j * BLK, row_vecs - 1));
 
     for (int g0 = 0; g0 < K; g0 += FAN) {
+      // (a later group waits for its ids inside the branch: a wait at the place where the two paths
+      // meet would cover the first group's row as well, which is requested behind its ids)
+      int own = own0;
+      if (g0 > 0) own = first_use(indices[i0 + min(g0 + (lane & (FAN - 1)), K - 1)]);
       int mine[FAN];
 #pragma unroll
       for (int g = 0; g < FAN; ++g) {
         const int i = i0 + min(g0 + g, K - 1);
-        mine[g] = composite(indices[i], i);
+        mine[g] = composite(__builtin_amdgcn_readlane(own, g), i);
       }
       int cnt[FAN];
 #pragma unroll
@@ -617,12 +662,12 @@ __global__ __launch_bounds__(BLK) void dispatch_fanout_wide_kernel(
       lds_barrier();
       if (wave == 0) {  // row h of 16 lanes adds up pair h of every wave
         const int h = lane >> 4, w = lane & 15;
-        int sum = w < NW ? part[w * PAIRS + h] : 0;
+        int sum = w < NW && h < PAIRS ? part[w * PAIRS + h] : 0;
         sum = dpp_add<0x111, 0xf>(sum);
         sum = dpp_add<0x112, 0xf>(sum);
         sum = dpp_add<0x114, 0xf>(sum);
         sum = dpp_add<0x118, 0xf>(sum);
-        if (w == 15) total[h] = sum;
+        if (w == 15 && h < PAIRS) total[h] = sum;
       }
       lds_barrier();
       // no third barrier: `part` is next written before a barrier that wave 0 only reaches after
@@ -648,7 +693,8 @@ __global__ __launch_bounds__(BLK) void dispatch_fanout_wide_kernel(
 #pragma unroll
         for (int gg = 0; gg < FAN; ++gg) mine_slot = gg == g ? slot[gg] : mine_slot;
         const int i = i0 + g0 + g;
-        const int m = f == 0 ? indices[i] : f == 1 ? rank : f == 2 ? t : f == 3 ? g0 + g : 0;
+        const int e = __shfl(own, g, 64);  // (lanes 0 .. FAN-1 of wave 0 are among the active ones)
+        const int m = f == 0 ? e : f == 1 ? rank : f == 2 ? t : f == 3 ? g0 + g : 0;
         send_meta[(size_t)mine_slot * META + f] = m;
         if (f == 0 && send_slot) send_slot[i] = mine_slot;
       }
@@ -1007,8 +1053,13 @@ __global__ __launch_bounds__(64 * ROWS) void dispatch_recv_kernel(
   // only groups that lie wholly below the bound: their rows can be read as they are
   const int hint_items = hint_rows / ROWS * chunks;
   if (W <= 64 && q < hint_items) {
-    const int my_count = lane < W ? min(max(recv_counts[lane], 0), capacity_rows) : 0;  // in flight with the rows
-    R = move(q, hint_rows, [&] { return min(wave_sum(my_count), capacity_rows); });
+    // The count travels with the rows: nothing touches the loaded value before the key and row
+    // loads have been issued (first_use).
+    const int raw_count = recv_counts[min(lane, W - 1)];
+    R = move(q, hint_rows, [&] {
+      const int my_count = lane < W ? min(max(first_use(raw_count), 0), capacity_rows) : 0;
+      return min(wave_sum(my_count), capacity_rows);
+    });
     q += movers;
   } else {
     R = min(sum_counts(recv_counts, W, capacity_rows), capacity_rows);
@@ -1204,7 +1255,8 @@ __global__ __launch_bounds__(64 * ROWS) void combine_send_kernel(
       }
 
       const int items = R * chunks, movers = (gridDim.x - W) * ROWS;
-      for (int q = (blockIdx.x - W) * ROWS + wave; q < items; q += movers) {
+      for (int qv = (blockIdx.x - W) * ROWS + wave; qv < items; qv += movers) {
+        const int q = __builtin_amdgcn_readfirstlane(qv);  // the same for every lane of a wave
         const int g = chunks == 1 ? q : q / chunks, c = q - g * chunks;
         const int base = c * (64 * NVW);
         const int le = __popcll(__ballot(incl <= g));
@@ -1215,9 +1267,12 @@ __global__ __launch_bounds__(64 * ROWS) void combine_send_kernel(
         int m = 0;
         if (c == 0 && lane < META) m = expert_meta[row * META + lane];
         WavePayload<V, NVW> p;
-        p.load(expert_y + row * row_vecs, base, row_vecs, lane);
+        p.load(unknown_origin(expert_y + row * row_vecs), base, row_vecs, lane);
+        // (the row is only used by the stores below, which depend on the slot: without this the
+        // compiler moves the loads down behind the plan's round trip)
+        issued_here();
         // the run starts are ascending in the source rank: the last one at or below j is ours
-        const int src = max(__popcll(__ballot(run[0] <= j)) - 1, 0);
+        const int src = max((int)__popcll(__ballot(run[0] <= j)) - 1, 0);
         const int slot = __builtin_amdgcn_readlane(run[1], src) + (j - __builtin_amdgcn_readlane(run[0], src));
         if (slot >= 0 && slot < capacity_rows) {
           p.template store<(MOE_A2A_NT_CSEND != 0)>(send_buf + (size_t)slot * row_vecs, base, row_vecs, lane);
@@ -1384,14 +1439,6 @@ struct PairAcc {
 // batch of the scan is loaded before the true row count R is known (the counts
 // are loaded at the same time); rows at or past R are ignored.
 
-// Compare-exchange of two (row, k) pairs by row.
-__device__ __forceinline__ void order_pair(int& ra, int& ka, int& rb, int& kb) {
-  const bool swap = rb < ra;
-  const int r = swap ? rb : ra, k = swap ? kb : ka;
-  rb = swap ? ra : rb; kb = swap ? ka : kb;
-  ra = r; ka = k;
-}
-
 // Long streams: every workgroup of a token scanning the whole arriving stream makes the meta
 // reads grow with tokens x rows. return_map_kernel turns the stream into a table first: one
 // thread per arriving row writes its row number at entry_row[src_token * K + src_k]. A token's
@@ -1433,8 +1480,13 @@ __global__ __launch_bounds__(BLK) void combine_recv_kernel(
   const int tid = threadIdx.x, lane = tid & 63;
   const int kw = min(K, COMBINE_WEIGHTS);
   const bool lanes_hold_counts = W <= 64;
-  const int my_count = lanes_hold_counts && lane < W ? min(max(recv_counts[lane], 0), capacity_rows) : 0;
+  // in flight with the first batch of the scan (first_use)
+  const int raw_count = recv_counts[min(lane, W - 1)];
   int R = -1;  // not known yet
+  auto rows_arrived = [&] {
+    const int my_count = lane < W ? min(max(first_use(raw_count), 0), capacity_rows) : 0;
+    return min(lanes_hold_counts ? wave_sum(my_count) : sum_counts(recv_counts, W, capacity_rows), capacity_rows);
+  };
 
   // rows [lo, hi) of the arriving stream: note the ones addressed to token t
   auto scan = [&](int t, int lo, int hi) {
@@ -1449,11 +1501,12 @@ __global__ __launch_bounds__(BLK) void combine_recv_kernel(
         key[u] = tk[0];
         kk[u] = tk[1];
       }
-      if (R < 0) R = min(lanes_hold_counts ? wave_sum(my_count) : sum_counts(recv_counts, W, capacity_rows), capacity_rows);
+      if (R < 0) R = rows_arrived();
 #pragma unroll
       for (int u = 0; u < SCAN_UNROLL; ++u) {
         const int row = b + tid + u * BLK;
-        if (row < min(hi, R) && key[u] == t) {
+        // (an arriving row whose k names no weight of the token is not an addend)
+        if (row < min(hi, R) && key[u] == t && (uint32_t)kk[u] < (uint32_t)K) {
           const int p = atomicAdd(&nhit, 1);
           if (p < COMBINE_CAP) {
             hit_row[p] = row;
@@ -1486,7 +1539,7 @@ __global__ __launch_bounds__(BLK) void combine_recv_kernel(
     if (tid == 0) nhit = 0;
     lds_barrier();
     if constexpr (MAPPED) {
-      if (R < 0) R = min(lanes_hold_counts ? wave_sum(my_count) : sum_counts(recv_counts, W, capacity_rows), capacity_rows);
+      if (R < 0) R = rows_arrived();
       for (int k = tid; k < K; k += BLK) {
         const int i = entry_row[(size_t)t * K + k];
         if ((uint32_t)i < (uint32_t)R) {
@@ -1505,7 +1558,7 @@ __global__ __launch_bounds__(BLK) void combine_recv_kernel(
       // first item: one batch below the readable bound goes out before R is known
       const int spec = min(hint_rows, SCAN_UNROLL * BLK);
       scan(t, 0, spec);
-      if (R < 0) R = min(lanes_hold_counts ? wave_sum(my_count) : sum_counts(recv_counts, W, capacity_rows), capacity_rows);
+      if (R < 0) R = rows_arrived();
       scan(t, spec, R);
     } else {
       scan(t, 0, R);
@@ -1514,39 +1567,42 @@ __global__ __launch_bounds__(BLK) void combine_recv_kernel(
     lds_barrier();
     const int n = nhit;
 
-    if (n <= FAST) {
-      // order the (at most 8) hits by arrival index in registers, every lane for itself
-      int hr[FAST], hk[FAST];
-#pragma unroll
-      for (int u = 0; u < FAST; ++u) {
-        hr[u] = u < n ? hit_row[u] : INT_MAX;
-        hk[u] = u < n ? hit_k[u] : -1;
-      }
-#define MOE_A2A_CE(a, b) order_pair(hr[a], hk[a], hr[b], hk[b])
-      MOE_A2A_CE(0, 1); MOE_A2A_CE(2, 3); MOE_A2A_CE(4, 5); MOE_A2A_CE(6, 7);
-      MOE_A2A_CE(0, 2); MOE_A2A_CE(1, 3); MOE_A2A_CE(4, 6); MOE_A2A_CE(5, 7);
-      MOE_A2A_CE(1, 2); MOE_A2A_CE(5, 6);
-      MOE_A2A_CE(0, 4); MOE_A2A_CE(1, 5); MOE_A2A_CE(2, 6); MOE_A2A_CE(3, 7);
-      MOE_A2A_CE(2, 4); MOE_A2A_CE(3, 5);
-      MOE_A2A_CE(1, 2); MOE_A2A_CE(3, 4); MOE_A2A_CE(5, 6);
-#undef MOE_A2A_CE
+    if (n <= FAST && K <= COMBINE_WEIGHTS) {  // (every weight of the token is in LDS)
       if (n > 0) {
+        // Order the (at most 8) hits by arrival index. Lane l of every wave takes hit l % 8; its
+        // place in the order is the number of hits that arrived earlier, counted with seven
+        // rotations of a 16-lane DPP row (lanes 8..15 of a row hold the same eight hits again, so
+        // rotating by 1..7 shows a lane every other hit once). Each lane then pushes its hit to
+        // the lane of its place, and the ordered rows and weights are read lane by lane into
+        // scalar registers. About 45 vector instructions per wave; a sorting network on the
+        // hits as uniform values becomes some 150 scalar instructions, and the sixteen waves of a
+        // compute unit share one scalar unit.
+        const int p = lane & (FAST - 1);
+        const int hr = p < n ? hit_row[p] : INT_MAX;
+        const int hk = p < n ? hit_k[p] : 0;  // (0 <= k < K: checked when the hit was noted)
+        const float hw = wts[hk];
+        int place = 0;
+#define MOE_A2A_ROT(S) place += (int)(__builtin_amdgcn_update_dpp(0, hr, 0x120 + S, 0xf, 0xf, false) < hr)
+        MOE_A2A_ROT(1); MOE_A2A_ROT(2); MOE_A2A_ROT(3); MOE_A2A_ROT(4); MOE_A2A_ROT(5); MOE_A2A_ROT(6); MOE_A2A_ROT(7);
+#undef MOE_A2A_ROT
+        // (lanes without a hit all get place n, which nothing reads)
+        const int to = ((lane & ~(FAST - 1)) | place) << 2;
+        const int ordered_row = __builtin_amdgcn_ds_permute(to, hr);
+        const int ordered_w = __builtin_amdgcn_ds_permute(to, __float_as_int(hw));
         V v[FAST][NV];
         float w[FAST];
 #pragma unroll
         for (int u = 0; u < FAST; ++u) {
-          const int k = hk[u];
-          const bool ok = (u < n) & (k >= 0) & (k < K);
-          if (!ok) hr[u] = -1;
-          w[u] = !ok ? 0.0f : k < kw ? wts[k] : weights[(size_t)t * K + k];
-          const int row = ok ? hr[u] : 0;  // row 0 exists: n > 0; loaded and not used
+          // row 0 exists (n > 0): loaded for the places past n and not used
+          const int row = u < n ? __builtin_amdgcn_readlane(ordered_row, u) : 0;
+          w[u] = __int_as_float(__builtin_amdgcn_readlane(ordered_w, u));
 #pragma unroll
           for (int j = 0; j < NV; ++j)
             v[u][j] = recv_buf[(size_t)row * row_vecs + min(base + j * BLK + tid, row_vecs - 1)];
         }
 #pragma unroll
         for (int u = 0; u < FAST; ++u) {
-          if (hr[u] >= 0) {
+          if (u < n) {
 #pragma unroll
             for (int j = 0; j < NV; ++j)
 #pragma unroll
