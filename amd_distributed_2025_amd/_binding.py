@@ -86,9 +86,10 @@ class CtypesBinding:
         _lib.call("moe_a2a_expert_scale", C.byref(shape), _ptr(expert_x), _ptr(expert_num_tokens), rows_hint,
                   _DT[expert_x.dtype], _DT[expert_y.dtype], _ptr(expert_y), C.c_void_p(stream))
 
-    def expert_gemm(self, shape, expert_x, expert_num_tokens, rows_hint, weights, expert_y, stream):
+    def expert_gemm(self, shape, expert_x, expert_num_tokens, rows_hint, weights, bias, expert_y, stream):
         _lib.call("moe_a2a_expert_gemm", C.byref(shape), _ptr(expert_x), _ptr(expert_num_tokens), rows_hint,
-                  _ptr(weights), _DT[expert_x.dtype], _ptr(expert_y), C.c_void_p(stream))
+                  _ptr(weights), _ptr(bias), weights.shape[2], weights.shape[1], _DT[expert_x.dtype],
+                  _ptr(expert_y), C.c_void_p(stream))
 
     def linear(self, input, weight, bias, output, stream):
         m, k = input.shape
@@ -145,9 +146,9 @@ class ExtBinding:
     def expert_scale(self, shape, expert_x, expert_num_tokens, rows_hint, expert_y, stream):
         self._m.a2a_expert_scale(self._shape(shape), expert_x, expert_num_tokens, rows_hint, expert_y, stream)
 
-    def expert_gemm(self, shape, expert_x, expert_num_tokens, rows_hint, weights, expert_y, stream):
-        self._m.a2a_expert_gemm(self._shape(shape), expert_x, expert_num_tokens, rows_hint, weights, expert_y,
-                                stream)
+    def expert_gemm(self, shape, expert_x, expert_num_tokens, rows_hint, weights, bias, expert_y, stream):
+        self._m.a2a_expert_gemm(self._shape(shape), expert_x, expert_num_tokens, rows_hint, weights, bias,
+                                expert_y, stream)
 
     def linear(self, input, weight, bias, output, stream):
         self._m.a2a_linear(input, weight, bias, output, stream)

@@ -47,7 +47,7 @@ SIGNATURES = {
     "moe_a2a_combine_recv": [_SP, _P, _P, _P, _I, _I, _P, _I, _P, _I, _I, _P],
     "moe_a2a_combine_recv_long": [_SP, _P, _P, _P, _I, _I, _P, _I, _P, _I, _I, _P, _P],
     "moe_a2a_expert_scale": [_SP, _P, _P, _I, _I, _I, _P, _P],
-    "moe_a2a_expert_gemm": [_SP, _P, _P, _I, _P, _I, _P, _P],
+    "moe_a2a_expert_gemm": [_SP, _P, _P, _I, _P, _P, _I, _I, _I, _P, _P],
     "moe_a2a_linear": [_P, _P, _P, _I, _I, _I, _I, _P, _P],
     "moe_a2a_exchange_local": [_I, _I, _P, _P, _P, _I, _P, _P, _P, _I, _I, _I, _I, _P],
 }

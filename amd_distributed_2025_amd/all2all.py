@@ -176,24 +176,48 @@ class HIPAllToAll:
         self.binding.expert_scale(self.shape, expert_x, expert_num_tokens, hint, ey, _stream(self.device))
         return ey
 
-    def expert_gemm(self, expert_x, expert_num_tokens, weights, rows_hint: Optional[int] = None):
-        """The expert computation as a grouped GEMM: `expert_x[le, j] @ weights[le].T` on the valid
-        rows, float32 accumulation, one rounding. `weights` is [nle, H, H] of the row type with the
-        input index contiguous. Takes the place of all2all/reference.py:262 in a model; needs
-        in_dtype == out_dtype and hidden_dim % 64 == 0."""
-        cfg = self.cfg
-        if cfg.in_dtype != cfg.out_dtype:
-            raise ValueError("expert_gemm computes in one 16-bit type: in_dtype must equal out_dtype")
-        nle = cfg.num_experts // self.world_size
-        _need(expert_x, cfg.in_dtype, self.device, "expert_x")
+    def expert_gemm(self, expert_x, expert_num_tokens, weights, bias=None, rows_hint: Optional[int] = None,
+                    out: Optional[torch.Tensor] = None):
+        """One linear layer of the expert as a grouped GEMM over the expert-major layout:
+        `expert_x[le, j] @ weights[le].T (+ bias[le])` on the valid rows, float32 accumulation, one
+        rounding (two with a bias, as `x @ w.T + b` on 16-bit tensors). Takes the place of
+        all2all/reference.py:262 in a model.
+
+        `expert_x` is [nle, max_recv, in_dim] (what `dispatch` returned, or the result of an earlier
+        layer), `weights` [nle, out_dim, in_dim] with the input index contiguous, `bias` [nle,
+        out_dim] or None, all of one 16-bit type; returns [nle, max_recv, out_dim] (a workspace
+        buffer per out_dim unless `out` is given; never the input's memory). Limits of the
+        kernels: out_dim % 32 == 0 and in_dim % 8 == 0."""
+        nle = self.num_local_experts
+        dt = expert_x.dtype
+        if dt not in _binding._DT:
+            raise TypeError(f"expert_x: expected a 16-bit float type, got {dt}")
+        _need(expert_x, dt, self.device, "expert_x")
         _need(expert_num_tokens, torch.int32, self.device, "expert_num_tokens")
-        _need(weights, cfg.in_dtype, self.device, "weights")
-        if tuple(weights.shape) != (nle, cfg.hidden_dim, cfg.hidden_dim):
-            raise ValueError(f"weights must be [{nle}, {cfg.hidden_dim}, {cfg.hidden_dim}], got {tuple(weights.shape)}")
+        _need(weights, dt, self.device, "weights")
+        if expert_x.dim() != 3 or tuple(expert_x.shape[:2]) != (nle, self.max_recv):
+            raise ValueError(f"expert_x must be [{nle}, {self.max_recv}, in_dim], got {tuple(expert_x.shape)}")
+        in_dim = expert_x.shape[2]
+        if weights.dim() != 3 or weights.shape[0] != nle or weights.shape[2] != in_dim:
+            raise ValueError(f"weights must be [{nle}, out_dim, {in_dim}], got {tuple(weights.shape)}")
+        out_dim = weights.shape[1]
+        if bias is not None:
+            _need(bias, dt, self.device, "bias")
+            if tuple(bias.shape) != (nle, out_dim):
+                raise ValueError(f"bias must be [{nle}, {out_dim}], got {tuple(bias.shape)}")
         hint = self._default_rows_in(rows_hint)
-        ey = self._buf("expert_y", tuple(expert_x.shape), cfg.out_dtype)
-        self.binding.expert_gemm(self.shape, expert_x, expert_num_tokens, hint, weights, ey, _stream(self.device))
-        return ey
+        if out is None:
+            name = f"expert_out_{out_dim}"
+            if name in self._ws and self._ws[name].data_ptr() == expert_x.data_ptr():
+                name += "_b"  # a layer of equal width reading the buffer the one before it wrote
+            out = self._buf(name, (nle, self.max_recv, out_dim), dt)
+        else:
+            _need(out, dt, self.device, "out")
+            if tuple(out.shape) != (nle, self.max_recv, out_dim) or out.data_ptr() == expert_x.data_ptr():
+                raise ValueError(f"out must be [{nle}, {self.max_recv}, {out_dim}] and not the input")
+        self.binding.expert_gemm(self.shape, expert_x, expert_num_tokens, hint, weights, bias, out,
+                                 _stream(self.device))
+        return out
 
     def combine_send(self, expert_meta, expert_y, expert_num_tokens, rows_hint: Optional[int] = None):
         """Expert-major results -> rows grouped by origin rank.
@@ -397,9 +421,15 @@ class LocalWorld:
             got.append((rc, rb, rm, total))
         return got
 
-    def run(self, rank_data: Sequence[RankTestData], accumulate: bool = False) -> List[torch.Tensor]:
+    def run(self, rank_data: Sequence[RankTestData], accumulate: bool = False,
+            expert: Optional[Callable] = None) -> List[torch.Tensor]:
         """`ref_kernel` (all2all/reference.py:256-272) for every rank; returns each
-        rank's `y[:num_tokens]`. Intermediates are kept in `self.trace[r]`."""
+        rank's `y[:num_tokens]`. Intermediates are kept in `self.trace[r]`.
+
+        `expert(rank_object, expert_x, expert_num_tokens, rows_hint)` returns the rank's
+        `expert_y [nle, max_recv, hidden_dim]` of `out_dtype`: what a model runs where the
+        reference has `expert_x.to(out_dtype) * (1 + rank)` (reference.py:262), for example layers
+        of `HIPAllToAll.expert_gemm`. None is the reference's stand-in."""
         cfg = self.cfg
         sent = []
         for r, a in enumerate(self.ranks):
@@ -412,7 +442,7 @@ class LocalWorld:
         for r, a in enumerate(self.ranks):
             rc, rb, rm, total = got[r]
             num, ex, em = a.dispatch_recv(rc, rb, rm, total)
-            ey = a.expert_scale(ex, num, total)
+            ey = a.expert_scale(ex, num, total) if expert is None else expert(a, ex, num, total)
             bc, bb, bm = a.combine_send(em, ey, num, total)
             back.append((bc, bb, bm))
             self.trace[r].update(recv_counts=rc, recv_buf=rb, recv_meta=rm, expert_num_tokens=num,

@@ -3231,11 +3231,12 @@ int launch_dense_gemm(const void* a, const void* b, const void* bias, void* c, i
 // rows that the matrix cores, not the stream of weights, bound the work, and the dense kernel's
 // tiles (each weight row read once per 128 or 256 rows, operands shared by four waves through
 // LDS) do better than the kernel that is built around streaming. MOE_A2A_NOT_DENSE otherwise.
-int launch_grouped_dense(const void* x, const int32_t* rows_of_group, const void* w, void* y, int groups,
-                         long long max_rows, long long rows_hint, int N, int K, int dtype, hipStream_t st) {
+int launch_grouped_dense(const void* x, const int32_t* rows_of_group, const void* w, const void* bias, void* y,
+                         int groups, long long max_rows, long long rows_hint, int N, int K, int dtype,
+                         hipStream_t st) {
   if (dtype != MOE_A2A_F16 && dtype != MOE_A2A_BF16) return MOE_A2A_EINVAL;
   if (N % 32 != 0 || K % 8 != 0) return MOE_A2A_EINVAL;
-  if (!all_aligned(16, x, w, y)) return MOE_A2A_EALIGN;
+  if (!all_aligned(16, x, w, y) || !all_aligned(8, bias)) return MOE_A2A_EALIGN;
   if (!rows_of_group || rows_hint < (long long)MOE_A2A_GROUPED_DENSE_MIN_ROWS * groups) return MOE_A2A_NOT_DENSE;
   if ((long long)K * 2 * 256 >= (1 << 30) || max_rows > INT_MAX / 2) return MOE_A2A_NOT_DENSE;
 #ifndef MOE_A2A_GROUPED_DENSE_TILE
@@ -3256,8 +3257,8 @@ int launch_grouped_dense(const void* x, const int32_t* rows_of_group, const void
   if (const int rc = allow_large_lds()) return rc;
 #define LAUNCH_GD(DT, TM, TN)                                                                 \
   dense_gemm_kernel<DT, 2, 2, TM, TN, true><<<grid, 256, lds_bytes, st>>>(                    \
-      (const b128*)x, (const b128*)w, nullptr, (uint16_t*)y, 0, N, K, 0, (int)tiles_n, rows_of_group, groups, \
-      (int)max_rows)
+      (const b128*)x, (const b128*)w, (const uint16_t*)bias, (uint16_t*)y, 0, N, K, 0, (int)tiles_n,        \
+      rows_of_group, groups, (int)max_rows)
   if (dtype == MOE_A2A_BF16) {
     if (tile == 256) LAUNCH_GD(MOE_A2A_BF16, 4, 4);
     else if (tile == 128) LAUNCH_GD(MOE_A2A_BF16, 2, 2);
@@ -3319,16 +3320,18 @@ extern "C" {
 
 int moe_a2a_expert_gemm(const moe_a2a_shape* s, const void* expert_x,
                         const int32_t* expert_num_tokens, int32_t rows_hint, const void* weights,
-                        int32_t dtype, void* expert_y, void* stream) {
-  if (!shape_ok(s) || rows_hint < 0 || !expert_x || !expert_num_tokens || !weights || !expert_y)
+                        const void* bias, int32_t in_dim, int32_t out_dim, int32_t dtype,
+                        void* expert_y, void* stream) {
+  if (!shape_ok(s) || rows_hint < 0 || in_dim < 1 || out_dim < 1 || !expert_x || !expert_num_tokens ||
+      !weights || !expert_y)
     return MOE_A2A_EINVAL;
   const int nle = s->num_experts / s->world_size;
   const long long max_recv = (long long)s->max_num_tokens * s->world_size;
-  const int dense = launch_grouped_dense(expert_x, expert_num_tokens, weights, expert_y, nle, max_recv, rows_hint,
-                                         s->hidden_dim, s->hidden_dim, dtype, (hipStream_t)stream);
+  const int dense = launch_grouped_dense(expert_x, expert_num_tokens, weights, bias, expert_y, nle, max_recv,
+                                         rows_hint, out_dim, in_dim, dtype, (hipStream_t)stream);
   if (dense != MOE_A2A_NOT_DENSE) return dense;
-  return launch_grouped_gemm(expert_x, expert_num_tokens, weights, nullptr, expert_y, nle, max_recv,
-                             rows_hint, s->hidden_dim, s->hidden_dim, dtype, (hipStream_t)stream);
+  return launch_grouped_gemm(expert_x, expert_num_tokens, weights, bias, expert_y, nle, max_recv, rows_hint,
+                             out_dim, in_dim, dtype, (hipStream_t)stream);
 }
 
 int moe_a2a_linear(const void* input, const void* weight, const void* bias, int32_t m, int32_t n,

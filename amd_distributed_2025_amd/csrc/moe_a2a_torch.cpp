@@ -206,17 +206,26 @@ void a2a_expert_scale(std::vector<int64_t> shape, torch::Tensor expert_x, torch:
 }
 
 void a2a_expert_gemm(std::vector<int64_t> shape, torch::Tensor expert_x, torch::Tensor expert_num_tokens,
-                     int64_t rows_hint, torch::Tensor weights, torch::Tensor expert_y, int64_t stream) {
+                     int64_t rows_hint, torch::Tensor weights, c10::optional<torch::Tensor> bias,
+                     torch::Tensor expert_y, int64_t stream) {
   const moe_a2a_shape s = shape_of(shape);
   const auto dt = rows_type(expert_x, "expert_x");
   const int64_t nle = s.world_size > 0 ? s.num_experts / s.world_size : 0;
   const int64_t padded = nle * s.max_num_tokens * s.world_size;
-  need(expert_x, "expert_x", dt, padded * s.hidden_dim);
-  need(expert_y, "expert_y", dt, padded * s.hidden_dim, &expert_x);
-  need(weights, "weights", dt, nle * s.hidden_dim * s.hidden_dim, &expert_x);
+  TORCH_CHECK(weights.dim() == 3 && weights.size(0) == nle, "weights must be [num_local_experts, out_dim, in_dim]");
+  const int64_t out_dim = weights.size(1), in_dim = weights.size(2);
+  need(expert_x, "expert_x", dt, padded * in_dim);
+  need(expert_y, "expert_y", dt, padded * out_dim, &expert_x);
+  need(weights, "weights", dt, nle * out_dim * in_dim, &expert_x);
   need(expert_num_tokens, "expert_num_tokens", torch::kInt32, nle, &expert_x);
+  const void* b = nullptr;
+  if (bias.has_value()) {
+    need(*bias, "bias", dt, nle * out_dim, &expert_x);
+    b = bias->data_ptr();
+  }
   status(moe_a2a_expert_gemm(&s, expert_x.data_ptr(), ints(expert_num_tokens), to_i32(rows_hint, "rows_hint"),
-                             weights.data_ptr(), dtype_code(dt), expert_y.data_ptr(), stream_of(stream)),
+                             weights.data_ptr(), b, to_i32(in_dim, "in_dim"), to_i32(out_dim, "out_dim"),
+                             dtype_code(dt), expert_y.data_ptr(), stream_of(stream)),
          "moe_a2a_expert_gemm");
 }
 

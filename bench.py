@@ -380,7 +380,7 @@ def main():
         times = []
         for i in range(12):
             ev[0].record()
-            ey = a.expert_gemm(ex, num, wts, R)
+            ey = a.expert_gemm(ex, num, wts, rows_hint=R)
             ev[1].record()
             ev[1].synchronize()
             if i >= 2:

@@ -305,44 +305,53 @@ int moe_a2a_expert_scale(const moe_a2a_shape* shape, const void* expert_x,
                          void* stream);
 
 /*
- * The expert computation between dispatch and combine as a grouped GEMM over the
- * expert-major layout: for every local expert le and every valid row
+ * The expert computation between dispatch and combine as a grouped linear layer
+ * over the expert-major layout: for every local expert le and every valid row
  * j < expert_num_tokens[le]
- *   expert_y[le, j, :] = expert_x[le, j, :] @ weights[le]^T
- * with float32 accumulation and one rounding to the 16-bit type. It fills the
- * place of all2all/reference.py:262, where the reference has the simulated
- * expert `expert_x.to(out_dtype) * (1 + rank)` (moe_a2a_expert_scale keeps that
- * arithmetic for parity with the reference; this is what a model would run
- * there).
+ *   expert_y[le, j, :] = expert_x[le, j, :] @ weights[le]^T (+ bias[le])
+ * It fills the place of all2all/reference.py:262, where the reference has the
+ * simulated expert `expert_x.to(out_dtype) * (1 + rank)` (moe_a2a_expert_scale
+ * keeps that arithmetic for parity with the reference; this is what a model
+ * runs there). An expert of several layers is several calls: hidden_dim ->
+ * intermediate with in_dim = hidden_dim, then intermediate -> hidden_dim with
+ * out_dim = hidden_dim, whose result moe_a2a_combine_send takes.
  *
- *   expert_x   [nle, max_recv, H], expert_num_tokens [nle] as moe_a2a_dispatch_recv
- *              leaves them (counts above max_recv are clamped)
- *   weights    [nle, H, H] of the same 16-bit type: weights[le][n][k] multiplies
- *              input element k into output element n (the layout of a linear
- *              layer's weight, input index contiguous)
- *   dtype      MOE_A2A_F16 or MOE_A2A_BF16: element type of all three
- *   expert_y   [nle, max_recv, H] out; rows at or past expert_num_tokens[le] are
- *              not written
+ *   expert_x   [nle, max_recv, in_dim], expert_num_tokens [nle]: for the first
+ *              layer what moe_a2a_dispatch_recv leaves (in_dim = hidden_dim);
+ *              counts above max_recv are clamped
+ *   weights    [nle, out_dim, in_dim] of the same 16-bit type: weights[le][n][k]
+ *              multiplies input element k into output element n (the layout of
+ *              a linear layer's weight, input index contiguous)
+ *   bias       [nle, out_dim] of the same type, or NULL
+ *   dtype      MOE_A2A_F16 or MOE_A2A_BF16: element type of all four
+ *   expert_y   [nle, max_recv, out_dim] out; rows at or past
+ *              expert_num_tokens[le] are not written
+ * Arithmetic: float32 accumulation and one rounding to the 16-bit type; a bias
+ * is then added to that rounded value in float32 and the sum rounded again,
+ * which is what `x @ w.T + b` on 16-bit tensors does (the same as
+ * moe_a2a_linear).
  * Rows are processed in blocks found from the device-side counts, so the work
  * follows the rows, not the experts. rows_hint (the rows the caller expects
  * over all experts) picks the kernel and sizes the launch, and changes no bit
- * of the result: from about 56 rows per expert, output tiles of 128 x 128
- * (64 x 128 when those would be too few for the GPU, 256 x 256 from about 768
- * rows per expert) of the kernel behind moe_a2a_linear, numbered over the
- * experts; below, a kernel built around streaming every weight once, in blocks
- * of 64 or 128 tokens and workgroups 128 to 256 columns wide. The first call on
- * a GPU sets kernel attributes (tiles can use more LDS than a kernel gets by
- * default): make that call outside a graph capture. Limits: hidden_dim a
- * multiple of 32, all three buffers 16-byte aligned (MOE_A2A_EINVAL / EALIGN).
+ * of the result: from 56 rows per expert on average, output tiles of 128 x 128
+ * (64 x 128 when those would be too few for the GPU, 256 x 256 from 768 rows
+ * per expert) of the kernel behind moe_a2a_linear, numbered over the experts;
+ * below, a kernel built around streaming every weight once, in blocks of 64 or
+ * 128 tokens and workgroups 128 to 256 columns wide. The first call on a GPU
+ * sets kernel attributes (tiles can use more LDS than a kernel gets by default):
+ * make that call outside a graph capture.
+ * Limits: out_dim a multiple of 32, in_dim a multiple of 8, expert_x / weights /
+ * expert_y 16-byte and bias 8-byte aligned (MOE_A2A_EINVAL / EALIGN).
  * Sums are formed in float32 in the order of the matrix unit, which is not the
  * order of a CPU matmul: results lie within what float32 accumulation in any
- * order plus one rounding allows around the exact product, and are exact when
+ * order plus the roundings allow around the exact value, and are exact when
  * every order gives the same float32 sum (identity and signed permutation
  * weights, small integers).
  */
 int moe_a2a_expert_gemm(const moe_a2a_shape* shape, const void* expert_x,
                         const int32_t* expert_num_tokens, int32_t rows_hint,
-                        const void* weights, int32_t dtype, void* expert_y,
+                        const void* weights, const void* bias, int32_t in_dim,
+                        int32_t out_dim, int32_t dtype, void* expert_y,
                         void* stream);
 
 /*

@@ -292,17 +292,61 @@ def combine_recv(
 # ----------------------------------------------------------------------------- whole job
 
 
+def grouped_linear(rows: np.ndarray, counts: np.ndarray, weights: np.ndarray, bias, dtype: str) -> np.ndarray:
+    """A linear layer per local expert over the compact expert-major rows: the rows of expert le
+    (`counts[le]` of them, experts back to back) go through `linear(rows, weights[le], bias[le])`.
+    `weights` is [nle, out_dim, in_dim], `bias` [nle, out_dim] or None, as bit patterns."""
+    out = np.empty((rows.shape[0], weights.shape[1]), np.uint16)
+    g = 0
+    for le, n in enumerate(int(c) for c in counts):
+        out[g:g + n] = linear(rows[g:g + n], weights[le], None if bias is None else bias[le], dtype)
+        g += n
+    return out
+
+
+def combine_bound(ret_exact: np.ndarray, ret_tol: np.ndarray, ret_meta: np.ndarray, weights: np.ndarray,
+                  num_rows_out: int, dtype: str):
+    """(exact, tol) for `combine_recv` when the arriving rows are only known to lie within
+    `ret_tol` of `ret_exact` (float64, e.g. from `linear_bound`): the float64 value of
+    sum_k w[t, k] * row and how far from it the 16-bit result of the per-addend-rounded
+    accumulation can lie. Per addend: the row's own distance times |w|, a half unit of the 16-bit
+    type on the value the row was rounded to before it was sent, the float32 product and sum
+    (2^-23 of the running magnitude) and the rounding of the accumulator (a half unit of the
+    running magnitude). The running magnitude is bounded by the sum of |w||row| so far plus the
+    error so far."""
+    u16, floor = (2.0 ** -8, 2.0 ** -133) if dtype == "bf16" else (2.0 ** -11, 2.0 ** -24)
+    H = ret_exact.shape[1]
+    exact = np.zeros((num_rows_out, H))
+    mass = np.zeros((num_rows_out, H))
+    tol = np.zeros((num_rows_out, H))
+    w_all = np.asarray(weights, dtype=np.float64)
+    for i in range(ret_meta.shape[0]):  # arrival order
+        t, k = int(ret_meta[i, 2]), int(ret_meta[i, 3])
+        w = abs(w_all[t, k])
+        exact[t] += w_all[t, k] * ret_exact[i]
+        mass[t] += w * np.abs(ret_exact[i])
+        tol[t] += w * ret_tol[i]
+        tol[t] += (u16 + 2.0 ** -22) * (mass[t] + tol[t]) + floor
+    return exact, tol
+
+
 def run_world(
     inputs: List[RankInput],
     num_experts: int,
     max_num_tokens: int,
     in_dtype: str = "bf16",
     out_dtype: str = "bf16",
+    expert=None,
 ) -> List[RankTrace]:
     """`ref_kernel` (all2all/reference.py:256-272) for every rank of one job.
 
     Returns one RankTrace per rank. `y` has `num_tokens` rows (the reference
-    returns `y[:num_tokens]`)."""
+    returns `y[:num_tokens]`).
+
+    `expert(rank, rows, counts)` stands where the reference has its simulated expert
+    (reference.py:262): it gets the rank's compact expert-major rows ([R, H] bit patterns of
+    `in_dtype`, the rows of local expert 0 first) and the rows per local expert, and returns
+    [R, H] bit patterns of `out_dtype`. None is the reference's `x.to(out_dtype) * (1 + rank)`."""
     W = len(inputs)
     nle = num_experts // W
     max_recv = max_num_tokens * W
@@ -322,7 +366,12 @@ def run_world(
         tr[r].expert_rows = tr[r].recv_buf[order]
         tr[r].expert_meta_rows = tr[r].recv_meta[order]
         tr[r].extra["local"], tr[r].extra["pos"] = local, pos
-        tr[r].expert_y_rows = expert_scale(tr[r].expert_rows, r, in_dtype, out_dtype)
+        if expert is None:
+            tr[r].expert_y_rows = expert_scale(tr[r].expert_rows, r, in_dtype, out_dtype)
+        else:
+            tr[r].expert_y_rows = np.ascontiguousarray(expert(r, tr[r].expert_rows, cnt), dtype=np.uint16)
+            if tr[r].expert_y_rows.shape != tr[r].expert_rows.shape:
+                raise ValueError("the expert must return one row of hidden_dim per row it was given")
         bc, border = return_order(tr[r].expert_meta_rows, W)
         tr[r].back_counts = bc
         tr[r].back_buf = tr[r].expert_y_rows[border]

@@ -26,9 +26,9 @@ def oracle_inputs(world):
     ]
 
 
-def run_oracle(world):
+def run_oracle(world, expert=None):
     from amd_distributed_2025_amd.task import dtype_name
 
     cfg = world[0][0]
     return orc.run_world(oracle_inputs(world), cfg.num_experts, cfg.max_num_tokens,
-                         dtype_name(cfg.in_dtype), dtype_name(cfg.out_dtype))
+                         dtype_name(cfg.in_dtype), dtype_name(cfg.out_dtype), expert=expert)

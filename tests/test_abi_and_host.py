@@ -115,13 +115,17 @@ def test_bad_arguments_are_rejected_without_touching_the_gpu():
     assert lib.moe_a2a_combine_recv(C.byref(ok), one, one, one, 4, -1, one, 4, one, 0, 1, None) == -1
     assert lib.moe_a2a_combine_recv(C.byref(ok), one, one, one, 4, 1 << 30, one, 4, one, 0, 1, None) == -1
     assert lib.moe_a2a_expert_scale(C.byref(ok), one, one, 4, 0, 5, one, None) == -1
-    # grouped GEMM: bad dtype, negative hint, null weights, hidden_dim not a multiple of 32, odd alignment
-    assert lib.moe_a2a_expert_gemm(C.byref(ok), one, one, 4, one, 2, one, None) == -1
-    assert lib.moe_a2a_expert_gemm(C.byref(ok), one, one, -1, one, 1, one, None) == -1
-    assert lib.moe_a2a_expert_gemm(C.byref(ok), one, one, 4, None, 1, one, None) == -1
-    assert lib.moe_a2a_expert_gemm(C.byref(_lib.Shape(8, 0, 256, 8, 7168 + 16, 256)), one, one, 4, one, 1, one,
-                                   None) == -1
-    assert lib.moe_a2a_expert_gemm(C.byref(ok), one, one, 4, C.c_void_p(24), 1, one, None) == -2
+    # grouped GEMM: bad dtype, negative hint, null weights, out_dim not a multiple of 32, in_dim not a
+    # multiple of 8, dims below 1, odd alignment of the weights and of the bias
+    assert lib.moe_a2a_expert_gemm(C.byref(ok), one, one, 4, one, None, 64, 64, 2, one, None) == -1
+    assert lib.moe_a2a_expert_gemm(C.byref(ok), one, one, -1, one, None, 64, 64, 1, one, None) == -1
+    assert lib.moe_a2a_expert_gemm(C.byref(ok), one, one, 4, None, None, 64, 64, 1, one, None) == -1
+    assert lib.moe_a2a_expert_gemm(C.byref(ok), one, one, 4, one, None, 64, 48, 1, one, None) == -1
+    assert lib.moe_a2a_expert_gemm(C.byref(ok), one, one, 4, one, None, 60, 64, 1, one, None) == -1
+    assert lib.moe_a2a_expert_gemm(C.byref(ok), one, one, 4, one, None, 0, 64, 1, one, None) == -1
+    assert lib.moe_a2a_expert_gemm(C.byref(ok), one, one, 4, one, None, 64, 0, 1, one, None) == -1
+    assert lib.moe_a2a_expert_gemm(C.byref(ok), one, one, 4, C.c_void_p(24), None, 64, 64, 1, one, None) == -2
+    assert lib.moe_a2a_expert_gemm(C.byref(ok), one, one, 4, one, C.c_void_p(20), 64, 64, 1, one, None) == -2
     # dense product: negative m, null weight, n not a multiple of 32, k not a multiple of 8, odd bias pointer
     assert lib.moe_a2a_linear(one, one, None, -1, 64, 64, 1, one, None) == -1
     assert lib.moe_a2a_linear(one, None, None, 4, 64, 64, 1, one, None) == -1

@@ -29,9 +29,9 @@ def run_gemm(a, ex, counts, w, hint=None):
     """Runs the kernel twice into the same buffer, the second time over a buffer of
     sentinels, and returns the bit patterns of that second result."""
     num = torch.tensor(counts, dtype=torch.int32, device=DEV)
-    ey = a.expert_gemm(ex, num, w, hint)
+    ey = a.expert_gemm(ex, num, w, rows_hint=hint)
     ey.view(torch.int16).fill_(SENTINEL)
-    again = a.expert_gemm(ex, num, w, hint)
+    again = a.expert_gemm(ex, num, w, rows_hint=hint)
     assert again.data_ptr() == ey.data_ptr()
     torch.cuda.synchronize()
     return bits(again)
@@ -97,6 +97,41 @@ def test_small_integers_sum_exactly(H, dt):
         assert np.array_equal(orc.b16_to_f32(orc.expert_gemm(bits(torch.from_numpy(x[le, :c]).to(dt)),
                                                              bits(torch.from_numpy(w[le]).to(dt)), name), name),
                               want.astype(np.float32))
+
+
+@pytest.mark.parametrize("dt", [torch.bfloat16, torch.float16], ids=["bf16", "fp16"])
+@pytest.mark.parametrize("in_dim,out_dim", [(96, 160), (200, 64), (128, 128)])
+def test_bias_and_unequal_widths_on_every_kernel(in_dim, out_dim, dt):
+    """[nle, out_dim, in_dim] weights with a bias, small integers (every order of the sum agrees, and
+    both roundings are exact): the streaming kernel (row count 0) and the tiles of 64 x 128 / 128 x 128
+    and 256 x 256 (row counts of 56 and 768 per expert) all give the integers of `x @ w.T + b`."""
+    print(f"bias in={in_dim} out={out_dim} {dt}", flush=True)
+    rng = np.random.default_rng(in_dim * 7 + out_dim)
+    W, nle, max_tokens = 1, 5, 300
+    a, cfg = rank_object(W, nle, in_dim, max_tokens, dt)
+    counts = ragged_counts(rng, nle, max_tokens, [max_tokens, 0, 65, 129])
+    x = rng.integers(-1, 2, (nle, max_tokens, in_dim))
+    w = rng.integers(-1, 2, (nle, out_dim, in_dim))
+    b = rng.integers(-20, 21, (nle, out_dim))
+    ex, wt, bt = (torch.from_numpy(v).to(dt).to(DEV) for v in (x, w, b))
+    num = torch.tensor(counts, dtype=torch.int32, device=DEV)
+    name = dtype_name(dt)
+    for hint in (0, 56 * nle, 768 * nle):
+        out = torch.empty(nle, max_tokens, out_dim, dtype=dt, device=DEV)
+        out.view(torch.int16).fill_(SENTINEL)
+        got = a.expert_gemm(ex, num, wt, bias=bt, rows_hint=hint, out=out)
+        assert got.data_ptr() == out.data_ptr()
+        torch.cuda.synchronize()
+        got = bits(got)
+        check_padding_untouched(got, counts)
+        for le, c in enumerate(counts):
+            want = x[le, :c] @ w[le].T + b[le][None, :]   # |values| <= 200 + 20: integers both types hold
+            assert np.array_equal(orc.b16_to_f32(got[le, :c], name), want.astype(np.float32)), f"hint {hint} expert {le}"
+    # the oracle's statement of the same layer
+    rows = np.concatenate([x[le, :c] for le, c in enumerate(counts)])
+    want = np.concatenate([x[le, :c] @ w[le].T + b[le][None, :] for le, c in enumerate(counts)])
+    stated = orc.grouped_linear(bits(torch.from_numpy(rows).to(dt)), np.array(counts), bits(wt.cpu()), bits(bt.cpu()), name)
+    assert np.array_equal(orc.b16_to_f32(stated, name), want.astype(np.float32))
 
 
 def random_case(a, cfg, W, counts, seed, hint=None, check_experts=None):
@@ -188,8 +223,10 @@ def test_unsupported_shapes_raise():
     w = torch.zeros(1, 80, 80, dtype=torch.bfloat16, device=DEV)
     with pytest.raises(Exception, match="invalid|argument"):
         a.expert_gemm(ex, torch.tensor([4], dtype=torch.int32, device=DEV), w)
-    with pytest.raises(ValueError, match="weights must be"):
-        a.expert_gemm(ex, torch.tensor([4], dtype=torch.int32, device=DEV), w[:, :64])
+    with pytest.raises(ValueError, match="weights must be"):  # in_dim of the weights is not the rows'
+        a.expert_gemm(ex, torch.tensor([4], dtype=torch.int32, device=DEV), w[:, :, :64].contiguous())
+    with pytest.raises(ValueError, match="bias must be"):
+        a.expert_gemm(ex, torch.tensor([4], dtype=torch.int32, device=DEV), w, bias=w[0, :1, :64].contiguous())
 
 
 @pytest.mark.parametrize("H,width", [(576, 5), (640, 6), (704, 7), (832, 8)])
@@ -268,7 +305,7 @@ def test_graph_replays_of_both_products_match_eager():
     outs = {}
 
     def step():
-        outs["tiles"] = a.expert_gemm(ex, num, w, sum(counts))
+        outs["tiles"] = a.expert_gemm(ex, num, w, rows_hint=sum(counts))
         outs["linear"] = gemm_rs.local_product(lin, out=lin_out)
 
     side = torch.cuda.Stream()
@@ -287,7 +324,7 @@ def test_graph_replays_of_both_products_match_eager():
         graph.replay()
         torch.cuda.synchronize()
         got_tiles, got_lin = outs["tiles"].clone(), outs["linear"].clone()
-        want_tiles = a.expert_gemm(ex, num, w, 0).clone()   # eager, the streaming kernel: the same bits
+        want_tiles = a.expert_gemm(ex, num, w, rows_hint=0).clone()   # eager, the streaming kernel: the same bits
         want_lin = gemm_rs.local_product(lin).clone()
         torch.cuda.synchronize()
         for le, c in enumerate(counts):

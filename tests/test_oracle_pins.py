@@ -339,3 +339,79 @@ def test_gemm_bound_holds_for_torch_and_catches_a_dropped_term():
     exact, tol = orc.expert_gemm_bound(_b(x), _b(sq), "bf16")
     wrong = _b((x.float() @ sq.float()).to(torch.bfloat16))
     assert (np.abs(orc.b16_to_f32(wrong, "bf16").astype(np.float64) - exact) > tol).mean() > 0.5
+
+
+@pytest.mark.parametrize("name,tdt", [("bf16", torch.bfloat16), ("fp16", torch.float16)])
+def test_linear_bound_with_a_bias_holds_for_torch_and_catches_a_wrong_bias(name, tdt):
+    g = torch.Generator().manual_seed(7)
+    x = torch.randn(29, 384, generator=g).to(tdt)
+    w = (torch.randn(40, 384, generator=g) / 384 ** 0.5).to(tdt)
+    b = torch.randn(40, generator=g).to(tdt)
+    exact, tol = orc.linear_bound(_b(x), _b(w), _b(b), name)
+    assert np.allclose(exact, x.double().numpy() @ w.double().numpy().T + b.double().numpy()[None, :], rtol=1e-13)
+    off = lambda t16: np.abs(orc.b16_to_f32(_b(t16), name).astype(np.float64) - exact)
+    # torch's two statements (two roundings), the oracle's restatement of them, and the same sum
+    # rounded once (a fused epilogue) all lie inside
+    twice = torch.matmul(x, w.T) + b
+    once = (x.float() @ w.float().T + b.float()).to(tdt)
+    assert (off(twice) <= tol).all() and (off(once) <= tol).all()
+    assert (np.abs(orc.b16_to_f32(orc.linear(_b(x), _b(w), _b(b), name), name).astype(np.float64) - exact) <= tol).all()
+    # no bias, the bias twice, the bias of the neighbouring column: most results leave the bound
+    plain = torch.matmul(x, w.T)
+    for wrong in (plain, plain + b + b, plain + torch.roll(b, 1)):
+        assert (off(wrong) > tol).mean() > 0.5
+    # and the bound without a bias is the product's own
+    e0, t0 = orc.linear_bound(_b(x), _b(w), None, name)
+    e1, t1 = orc.expert_gemm_bound(_b(x), _b(w), name)
+    assert np.array_equal(e0, e1) and np.array_equal(t0, t1)
+
+
+def test_grouped_linear_is_a_linear_layer_per_expert():
+    g = torch.Generator().manual_seed(8)
+    counts = np.array([3, 0, 5, 1])
+    rows = torch.from_numpy(RNG.integers(-3, 4, (int(counts.sum()), 16))).to(torch.bfloat16)
+    w = torch.from_numpy(RNG.integers(-2, 3, (4, 24, 16))).to(torch.bfloat16)
+    b = torch.from_numpy(RNG.integers(-5, 6, (4, 24))).to(torch.bfloat16)
+    got = orc.grouped_linear(_b(rows), counts, _b(w), _b(b), "bf16")
+    start = 0
+    for le, c in enumerate(counts):  # small integers: exact in every order, so torch's result is THE result
+        want = torch.matmul(rows[start:start + c], w[le].T) + b[le]
+        assert np.array_equal(got[start:start + c], _b(want)), le
+        start += c
+    assert got.shape == (int(counts.sum()), 24)
+    assert np.array_equal(orc.grouped_linear(_b(rows), counts, _b(w), None, "bf16")[:3], _b(torch.matmul(rows[:3], w[0].T)))
+
+
+@pytest.mark.parametrize("name", ["bf16", "fp16"])
+def test_combine_bound_holds_and_catches_a_dropped_addend(name):
+    tdt = torch.bfloat16 if name == "bf16" else torch.float16
+    T, K, H = 6, 8, 96
+    g = torch.Generator().manual_seed(9)
+    rows16 = torch.randn(T * K, H, generator=g).to(tdt)
+    weights = torch.softmax(torch.randn(T, K, generator=g), dim=1).numpy()
+    order = RNG.permutation(T * K)  # arrival order of the (token, k) pairs
+    meta = np.zeros((T * K, 5), np.int32)
+    meta[:, 2], meta[:, 3] = order // K, order % K
+    exact_rows = rows16.double().numpy()
+    got = orc.combine_recv(_b(rows16), meta, weights, T, name)
+    exact, tol = orc.combine_bound(exact_rows, np.zeros_like(exact_rows), meta, weights, T, name)
+    want = np.zeros((T, H))
+    for i in range(T * K):
+        want[meta[i, 2]] += float(weights[meta[i, 2], meta[i, 3]]) * exact_rows[i]
+    assert np.allclose(exact, want, rtol=1e-12, atol=1e-300)
+    err = np.abs(orc.b16_to_f32(got, name).astype(np.float64) - exact)
+    assert (err <= tol).all()
+    assert (tol <= 0.05 * np.abs(exact).max()).all()  # (a bound that allowed everything would pin nothing)
+    # rows that are only known to within a tolerance: the result of any rows inside it stays inside
+    wiggle = 2.0 ** -7 * np.abs(exact_rows)
+    moved = torch.from_numpy(exact_rows * (1 + 2.0 ** -7 * RNG.choice([-1.0, 1.0], exact_rows.shape))).to(tdt)
+    _, tol_w = orc.combine_bound(exact_rows, wiggle * 1.02 + 2.0 ** -8 * np.abs(exact_rows), meta, weights, T, name)
+    err_w = np.abs(orc.b16_to_f32(orc.combine_recv(_b(moved), meta, weights, T, name), name).astype(np.float64) - exact)
+    assert (err_w <= tol_w).all()
+    # one addend of every token left out, and the weights of two k swapped: outside the bound
+    keep = np.ones(T * K, bool)
+    keep[[int(np.nonzero(meta[:, 2] == t)[0][3]) for t in range(T)]] = False
+    short = orc.combine_recv(_b(rows16)[keep], meta[keep], weights, T, name)
+    assert (np.abs(orc.b16_to_f32(short, name).astype(np.float64) - exact) > tol).mean() > 0.5
+    swapped = orc.combine_recv(_b(rows16), meta, weights[:, ::-1].copy(), T, name)
+    assert (np.abs(orc.b16_to_f32(swapped, name).astype(np.float64) - exact) > tol).mean() > 0.5
