@@ -103,6 +103,22 @@ class CtypesBinding:
                   rows_hint, _rows(send_buf, send_meta, hidden_dim), _rows(recv_buf, recv_meta, hidden_dim),
                   C.c_void_p(stream))
 
+    def gather_sources(self, hidden_dim, send_bufs, send_metas, send_counts):
+        """The per-source pointer tables of `exchange_gather`, built once for buffers that stay where
+        they are (a workspace): (tables, rows every send buffer holds, the tensors kept alive)."""
+        table = C.c_void_p * len(send_bufs)
+        return ((table(*[t.data_ptr() for t in send_bufs]), table(*[t.data_ptr() for t in send_metas]),
+                 table(*[t.data_ptr() for t in send_counts])),
+                min(_rows(b, m, hidden_dim) for b, m in zip(send_bufs, send_metas)),
+                (list(send_bufs), list(send_metas), list(send_counts)))
+
+    def exchange_gather(self, world_size, hidden_dim, sources, dst_rank, recv_buf, recv_meta, recv_counts,
+                        rows_hint, stream):
+        (bufs, metas, counts), send_capacity, _ = sources
+        _lib.call("moe_a2a_exchange_gather_local", world_size, hidden_dim, bufs, metas, counts, dst_rank,
+                  _ptr(recv_buf), _ptr(recv_meta), _ptr(recv_counts), rows_hint, send_capacity,
+                  _rows(recv_buf, recv_meta, hidden_dim), C.c_void_p(stream))
+
 
 class ExtBinding:
     name = "ext"
@@ -157,6 +173,15 @@ class ExtBinding:
                        recv_meta, recv_counts, src_rank, rows_hint, stream):
         self._m.a2a_exchange_local(world_size, hidden_dim, send_buf, send_meta, send_counts, dst_rank, recv_buf,
                                    recv_meta, recv_counts, src_rank, rows_hint, stream)
+
+    def gather_sources(self, hidden_dim, send_bufs, send_metas, send_counts):
+        return (list(send_bufs), list(send_metas), list(send_counts))
+
+    def exchange_gather(self, world_size, hidden_dim, sources, dst_rank, recv_buf, recv_meta, recv_counts,
+                        rows_hint, stream):
+        bufs, metas, counts = sources
+        self._m.a2a_exchange_gather_local(world_size, hidden_dim, bufs, metas, counts, dst_rank, recv_buf,
+                                          recv_meta, recv_counts, rows_hint, stream)
 
 
 _BINDINGS = {}

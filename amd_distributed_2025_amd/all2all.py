@@ -107,6 +107,12 @@ class HIPAllToAll:
                 self._buf("ret_buf", (self.max_rows_out, H), self.cfg.out_dtype),
                 self._buf("ret_meta", (self.max_rows_out, META_DIM), torch.int32))
 
+    def outbound_buffers(self, phase: str):
+        """What this rank's send half of `phase` wrote, as the whole workspace tensors (the send
+        halves return views cut to the rows in use): (counts[W], buf, meta)."""
+        names = ("send_counts", "send_buf", "send_meta") if phase == "dispatch" else ("back_counts", "back_buf", "back_meta")
+        return tuple(self._ws[n] for n in names)
+
     # ------------------------------------------------------------------ halves
 
     def dispatch_send(self, dp_x: torch.Tensor, indices: torch.Tensor, want_slots: bool = False):
@@ -153,7 +159,10 @@ class HIPAllToAll:
         _need(recv_buf, cfg.in_dtype, self.device, "recv_buf")
         _need(recv_meta, torch.int32, self.device, "recv_meta")
         capacity = min(recv_buf.shape[0], recv_meta.shape[0])
-        hint = min(capacity, self.max_rows_in if rows_hint is None else int(rows_hint))
+        # without a count from the caller: what balanced routing delivers (every rank sends its
+        # max_num_tokens * K rows and receives as many). A hint only sizes launches and picks the
+        # entry point; the kernels move whatever the device-side counts say.
+        hint = min(capacity, self.max_rows_out if rows_hint is None else int(rows_hint))
         nle = self.num_local_experts
         num = self._buf("expert_num_tokens", (nle,), torch.int32)
         ex = self._buf("expert_x", (nle, self.max_recv, cfg.hidden_dim), cfg.in_dtype)
@@ -271,7 +280,7 @@ class HIPAllToAll:
     def _default_rows_in(self, rows_hint):
         if rows_hint is not None:
             return int(rows_hint)
-        return int(getattr(self, "_rows_in_hint", self.max_rows_in))
+        return int(getattr(self, "_rows_in_hint", min(self.max_rows_in, self.max_rows_out)))
 
     # ------------------------------------------------------------------ reference surface
 
@@ -300,6 +309,23 @@ def exchange_leg(src: HIPAllToAll, dst: HIPAllToAll, send_counts, send_buf, send
     rows the four buffers were allocated with, whatever the counts say."""
     src.binding.exchange_local(src.world_size, src.cfg.hidden_dim, send_buf, send_meta, send_counts, dst.rank,
                                recv_buf, recv_meta, recv_counts, src.rank, int(rows_hint), _stream(src.device))
+
+
+GATHER_MAX_RANKS = 64  # source ranks one launch of moe_a2a_exchange_gather_local serves
+
+
+def gather_sources(ranks: Sequence[HIPAllToAll], phase: str):
+    """The source side of `exchange_gather` for all ranks of a job (whose send halves of `phase`
+    have run at least once, so that their workspaces exist); stays valid while those do."""
+    out = [a.outbound_buffers(phase) for a in ranks]
+    a0 = ranks[0]
+    return a0.binding.gather_sources(a0.cfg.hidden_dim, [o[1] for o in out], [o[2] for o in out], [o[0] for o in out])
+
+
+def exchange_gather(dst: HIPAllToAll, sources, recv_counts, recv_buf, recv_meta, rows_hint: int) -> None:
+    """Everything the ranks of a job hold for `dst`, counts included, in one launch."""
+    dst.binding.exchange_gather(dst.world_size, dst.cfg.hidden_dim, sources, dst.rank, recv_buf, recv_meta,
+                                recv_counts, int(rows_hint), _stream(dst.device))
 
 
 class LocalExchange:
@@ -336,14 +362,22 @@ class LocalExchange:
         self._barrier.wait()  # every rank has launched its send half
         posted = list(self._posted)
         rc, rb, rm = a.inbound_buffers(phase)
-        sent_here = torch.stack([p[1] for p in posted])[:, a.rank]  # rows each source holds for this rank
-        rc.copy_(sent_here)
-        host = sent_here.cpu().tolist() if self.exact_hints else None
         bound = min(rb.shape[0], rm.shape[0])
-        for s, (src, sc, sb, sm) in enumerate(posted):
-            hint = host[s] if host is not None else min(bound, sb.shape[0])
-            if hint > 0:
-                exchange_leg(src, a, sc, sb, sm, rc, rb, rm, hint)
+        if W <= GATHER_MAX_RANKS:
+            # one launch copies every source's segment and delivers the counts
+            host = None
+            if self.exact_hints:
+                host = torch.stack([p[1] for p in posted])[:, a.rank].cpu().tolist()
+            per_source = max(host) if host is not None else min(bound, max(1, 2 * a.max_rows_out // W))
+            exchange_gather(a, gather_sources([p[0] for p in posted], phase), rc, rb, rm, per_source)
+        else:
+            sent_here = torch.stack([p[1] for p in posted])[:, a.rank]  # rows each source holds for this rank
+            rc.copy_(sent_here)
+            host = sent_here.cpu().tolist() if self.exact_hints else None
+            for s, (src, sc, sb, sm) in enumerate(posted):
+                hint = host[s] if host is not None else min(bound, sb.shape[0])
+                if hint > 0:
+                    exchange_leg(src, a, sc, sb, sm, rc, rb, rm, hint)
         self._barrier.wait()  # every copy out of every send buffer has been launched
         return rc, rb, rm, (sum(host) if host is not None else None)
 
@@ -396,27 +430,41 @@ class LocalWorld:
         # replaying the same job without touching the host (graph capture)
         self.exact_hints = exact_hints
         self._last_counts = {}
+        self._sources = {}  # phase -> the source tables of the gathering exchange
         self.trace: List[dict] = [dict() for _ in range(world_size)]
 
     def _exchange(self, phase: str, sent: List[Tuple[torch.Tensor, torch.Tensor, torch.Tensor]]):
         W = self.world_size
-        all_counts = torch.stack([s[0] for s in sent])      # [src, dst]
-        per_dst = all_counts.t().contiguous()                # [dst, src]
-        bound = sent[0][1].shape[0]
         if self.exact_hints == "last":  # the counts read back by the previous run of the same job
             host = self._last_counts[phase]
         else:
-            host = all_counts.cpu().tolist() if self.exact_hints else None
+            host = torch.stack([s[0] for s in sent]).cpu().tolist() if self.exact_hints else None  # [src][dst]
             self._last_counts[phase] = host
         got = []
+        if W <= GATHER_MAX_RANKS:
+            # one launch per destination copies every source's segment and delivers the counts
+            sources = self._sources.get(phase)
+            if sources is None:  # (the workspaces the tables point into live as long as the ranks)
+                sources = self._sources[phase] = gather_sources(self.ranks, phase)
+            loose = max(1, 2 * self.ranks[0].max_rows_out // W)
+            for r, dst in enumerate(self.ranks):
+                rc, rb, rm = dst.inbound_buffers(phase)
+                per_source = max(host[s][r] for s in range(W)) if host is not None else loose
+                exchange_gather(dst, sources, rc, rb, rm, min(per_source, rb.shape[0]))
+                # (with "last" these are an earlier run's counts: they size launches and are no
+                # statement about this run)
+                got.append((rc, rb, rm, sum(host[s][r] for s in range(W)) if host is not None else None))
+            return got
+        per_dst = torch.stack([s[0] for s in sent]).t().contiguous()  # [dst, src]
+        bound = sent[0][1].shape[0]
         for r, dst in enumerate(self.ranks):
             rc, rb, rm = dst.inbound_buffers(phase)
             rc.copy_(per_dst[r])
             for s, src in enumerate(self.ranks):
                 hint = host[s][r] if host is not None else min(bound, sent[s][1].shape[0])
-                if host is not None and hint == 0:
+                if host is not None and hint == 0 and self.exact_hints != "last":
                     continue  # the counts were read back: this leg is known to be empty
-                exchange_leg(src, dst, sent[s][0], sent[s][1], sent[s][2], rc, rb, rm, hint)
+                exchange_leg(src, dst, sent[s][0], sent[s][1], sent[s][2], rc, rb, rm, max(hint, 1))
             total = sum(host[s][r] for s in range(W)) if host is not None else None
             got.append((rc, rb, rm, total))
         return got

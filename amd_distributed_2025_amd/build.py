@@ -28,7 +28,8 @@ EXT_DIR = PKG_DIR / "_ext"
 EXT_NAME = "moe_a2a_torch"
 # the wrappers load_inline binds, one per entry point of the C ABI
 EXT_FUNCTIONS = ["a2a_version", "a2a_dispatch_send", "a2a_plan_send", "a2a_dispatch_recv", "a2a_combine_send",
-                 "a2a_combine_recv", "a2a_expert_scale", "a2a_expert_gemm", "a2a_linear", "a2a_exchange_local"]
+                 "a2a_combine_recv", "a2a_expert_scale", "a2a_expert_gemm", "a2a_linear", "a2a_exchange_local",
+                 "a2a_exchange_gather_local"]
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950",

@@ -2506,6 +2506,50 @@ __global__ __launch_bounds__(BLOCK) void exchange_local_kernel(
   }
 }
 
+// All source legs of one destination in one launch: blockIdx.y is the source rank. The W source
+// buffers are separate allocations (one per rank object), so their addresses travel by value in
+// the kernel arguments. Every wave works out both offsets of its leg from the W counts the
+// sources hold for this destination (one lane per source, a wave scan) and the kernel also
+// writes those counts to recv_counts, which an exchange of counts would have delivered
+// (all2all/reference.py:88-91,181-185).
+constexpr int GATHER_MAX_RANKS = 64;
+struct GatherSources {
+  const void* buf[GATHER_MAX_RANKS];
+  const int* meta[GATHER_MAX_RANKS];
+  const int* counts[GATHER_MAX_RANKS];
+};
+
+template <typename V, int NV>
+__global__ __launch_bounds__(BLOCK) void exchange_gather_kernel(
+    GatherSources src, int W, int dst_rank, V* __restrict__ recv_buf, int* __restrict__ recv_meta,
+    int* __restrict__ recv_counts, int row_vecs, int chunks, int send_capacity_rows,
+    int recv_capacity_rows) {
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int s = blockIdx.y;
+  // rows every source holds for this destination (lane l: source l)
+  const int held = lane < W ? min(max(src.counts[lane][dst_rank], 0), send_capacity_rows) : 0;
+  const int upto = wave_inclusive_scan(held);
+  if (blockIdx.x == 0 && s == 0 && tid < W) recv_counts[tid] = held;
+  const int dst_off = __builtin_amdgcn_readlane(upto - held, s);
+  const int* __restrict__ my_counts = src.counts[s];
+  const int src_off = sum_counts(my_counts, dst_rank, send_capacity_rows);
+  int n = __builtin_amdgcn_readlane(held, s);
+  // never past what either buffer holds, whatever the counts claim
+  n = max(min(n, min(send_capacity_rows - src_off, recv_capacity_rows - dst_off)), 0);
+  const V* __restrict__ send_buf = (const V*)src.buf[s];
+  const int* __restrict__ send_meta = src.meta[s];
+  const int items = n * chunks;
+  for (int q = blockIdx.x; q < items; q += gridDim.x) {
+    const int i = chunks == 1 ? q : q / chunks, c = q - i * chunks;
+    const int base = c * (BLOCK * NV);
+    Payload<V, NV> p;
+    p.load(send_buf + (size_t)(src_off + i) * row_vecs, base, row_vecs);
+    p.store(recv_buf + (size_t)(dst_off + i) * row_vecs, base, row_vecs);
+    if (c == 0 && tid < META)
+      recv_meta[(size_t)(dst_off + i) * META + tid] = send_meta[(size_t)(src_off + i) * META + tid];
+  }
+}
+
 // ---------------------------------------------------------------- host side
 
 struct Geometry {
@@ -3372,5 +3416,44 @@ int moe_a2a_exchange_local(int32_t world_size, int32_t hidden_dim, const void* s
 #undef LAUNCH
   return launch_status();
 }
+
+int moe_a2a_exchange_gather_local(int32_t world_size, int32_t hidden_dim, const void* const* send_bufs,
+                                  const int32_t* const* send_metas, const int32_t* const* send_counts,
+                                  int32_t dst_rank, void* recv_buf, int32_t* recv_meta,
+                                  int32_t* recv_counts, int32_t rows_hint, int32_t send_capacity_rows,
+                                  int32_t recv_capacity_rows, void* stream) {
+  if (world_size < 1 || world_size > GATHER_MAX_RANKS || hidden_dim < 1 || dst_rank < 0 ||
+      dst_rank >= world_size || rows_hint < 0 || send_capacity_rows < 0 || recv_capacity_rows < 0 ||
+      !send_bufs || !send_metas || !send_counts || !recv_counts ||
+      !counts_fit(send_capacity_rows, world_size) || !counts_fit(recv_capacity_rows, world_size))
+    return MOE_A2A_EINVAL;
+  GatherSources src{};
+  bool all16 = aligned(recv_buf, 16);
+  for (int r = 0; r < world_size; ++r) {
+    if (!send_counts[r]) return MOE_A2A_EINVAL;
+    if (send_capacity_rows > 0 && (!send_bufs[r] || !send_metas[r])) return MOE_A2A_EINVAL;
+    if (!aligned(send_bufs[r], 2)) return MOE_A2A_EALIGN;
+    all16 = all16 && aligned(send_bufs[r], 16);
+    src.buf[r] = send_bufs[r];
+    src.meta[r] = send_metas[r];
+    src.counts[r] = send_counts[r];
+  }
+  if (send_capacity_rows > 0 && recv_capacity_rows > 0 && (!recv_buf || !recv_meta)) return MOE_A2A_EINVAL;
+  if (!aligned(recv_buf, 2)) return MOE_A2A_EALIGN;
+  Geometry g{};
+  row_geometry(g, hidden_dim, all16);
+  if (!items_fit(rows_hint, g.chunks)) return MOE_A2A_EINVAL;
+  // (the launch also delivers the counts, so it is made even when no row can move)
+  const dim3 grid(std::min(mover_blocks((long long)rows_hint * g.chunks), 1 << 16), world_size);
+  hipStream_t st = (hipStream_t)stream;
+#define LAUNCH(V, NV)                                                                          \
+  exchange_gather_kernel<V, NV><<<grid, BLOCK, 0, st>>>(src, world_size, dst_rank, (V*)recv_buf, \
+                                                        recv_meta, recv_counts, g.row_vecs, g.chunks, \
+                                                        send_capacity_rows, recv_capacity_rows)
+  MOE_A2A_FOR_ROW_KERNEL(g, LAUNCH);
+#undef LAUNCH
+  return launch_status();
+}
+
 
 }  // extern "C"

@@ -271,3 +271,37 @@ void a2a_exchange_local(int64_t world_size, int64_t hidden_dim, torch::Tensor se
                                 to_i32(recv_capacity, "recv_capacity_rows"), stream_of(stream)),
          "moe_a2a_exchange_local");
 }
+
+void a2a_exchange_gather_local(int64_t world_size, int64_t hidden_dim, std::vector<torch::Tensor> send_bufs,
+                               std::vector<torch::Tensor> send_metas, std::vector<torch::Tensor> send_counts,
+                               int64_t dst_rank, torch::Tensor recv_buf, torch::Tensor recv_meta,
+                               torch::Tensor recv_counts, int64_t rows_hint, int64_t stream) {
+  TORCH_CHECK(world_size >= 1 && world_size <= 64, "world_size: 1 to 64 source ranks in one launch");
+  TORCH_CHECK((int64_t)send_bufs.size() == world_size && (int64_t)send_metas.size() == world_size &&
+              (int64_t)send_counts.size() == world_size, "one send_buf, send_meta and send_counts per source rank");
+  const auto dt = rows_type(recv_buf, "recv_buf");
+  need(recv_buf, "recv_buf", dt, 0);
+  need(recv_meta, "recv_meta", torch::kInt32, 0, &recv_buf);
+  need(recv_counts, "recv_counts", torch::kInt32, world_size, &recv_buf);
+  const int64_t h = std::max<int64_t>(hidden_dim, 1);
+  const void* bufs[64];
+  const int32_t* metas[64];
+  const int32_t* counts[64];
+  int64_t send_capacity = INT32_MAX;
+  for (int64_t r = 0; r < world_size; ++r) {
+    need(send_bufs[r], "send_bufs[r]", dt, 0, &recv_buf);
+    need(send_metas[r], "send_metas[r]", torch::kInt32, 0, &recv_buf);
+    need(send_counts[r], "send_counts[r]", torch::kInt32, world_size, &recv_buf);
+    send_capacity = std::min(send_capacity, std::min(send_bufs[r].numel() / h, send_metas[r].numel() / MOE_A2A_META_DIM));
+    bufs[r] = send_bufs[r].data_ptr();
+    metas[r] = ints(send_metas[r]);
+    counts[r] = ints(send_counts[r]);
+  }
+  const int64_t recv_capacity = std::min(recv_buf.numel() / h, recv_meta.numel() / MOE_A2A_META_DIM);
+  status(moe_a2a_exchange_gather_local(to_i32(world_size, "world_size"), to_i32(hidden_dim, "hidden_dim"), bufs,
+                                       metas, counts, to_i32(dst_rank, "dst_rank"), recv_buf.data_ptr(),
+                                       ints(recv_meta), ints(recv_counts), to_i32(rows_hint, "rows_hint"),
+                                       to_i32(send_capacity, "send_capacity_rows"),
+                                       to_i32(recv_capacity, "recv_capacity_rows"), stream_of(stream)),
+         "moe_a2a_exchange_gather_local");
+}

@@ -82,6 +82,16 @@ def parse_args():
                          "(default: the host class's own threshold)")
     ap.add_argument("--alone", action="store_true",
                     help="also time every kernel back to back with itself (warm inputs)")
+    ap.add_argument("--dtype", default=None, choices=["fp16", "bf16"],
+                    help="token type of the main workload (default: the workload's own, bf16; the reference "
+                         "uses fp16, all2all/reference.py:16-17)")
+    ap.add_argument("--weights", default=None, choices=["rand", "softmax"],
+                    help="routing weights of the main workload (default: the workload's own, softmax; the "
+                         "reference draws rand, all2all/reference.py:37-43)")
+    ap.add_argument("--binding", default="ctypes", choices=["ctypes", "ext"],
+                    help="how the host class reaches the C ABI: ctypes, or the torch extension built with load_inline")
+    ap.add_argument("--no-extra-workloads", action="store_true",
+                    help="skip the C5 block and the C4 block with the reference's input rules (fp16, rand weights)")
     return ap.parse_args()
 
 
@@ -132,23 +142,32 @@ def main():
     torch.cuda.set_device(dev)
 
     from amd_distributed_2025_amd.task import LARGE_WORKLOADS
-    wl = {**WORKLOADS, **LARGE_WORKLOADS}[args.workload]
-    world = generate_world(wl, args.seed)
-    cfg = world[0][0]
+    wl = dict({**WORKLOADS, **LARGE_WORKLOADS}[args.workload])
+    if args.dtype:
+        wl["dtype"] = args.dtype
+    if args.weights:
+        wl["weights"] = args.weights
+
+    def set_up(workload):
+        """The whole job once, so that every rank's inbound buffers hold the peers' segments."""
+        world_ = generate_world(workload, args.seed)
+        cfg_ = world_[0][0]
+        data_ = [d.to(dev) for _, d, _, _ in world_]
+        lw_ = LocalWorld(cfg_, len(world_), device=dev, reuse_placement=not args.no_placement_plan,
+                         long_stream_rows=args.long_stream_rows, binding=args.binding)
+        ys_ = [y.clone() for y in lw_.run(data_)]
+        torch.cuda.synchronize()
+        return world_, cfg_, data_, lw_, ys_
+
+    world, cfg, data, lw, ys0 = set_up(wl)
     W, K, H = len(world), cfg.experts_per_token, cfg.hidden_dim
-    data = [d.to(dev) for _, d, _, _ in world]
     if not 0 <= args.rank < W:
         print(f"--rank must be in [0, {W})", file=sys.stderr)
         sys.exit(2)
 
-    # ---- set-up: the whole job once, so every rank's inbound buffers hold the peers' segments
-    lw = LocalWorld(cfg, W, device=dev, reuse_placement=not args.no_placement_plan,
-                    long_stream_rows=args.long_stream_rows)
-    ys0 = [y.clone() for y in lw.run(data)]
-    torch.cuda.synchronize()
-
-    def stages_of(r):
+    def stages_of(r, lw=lw, data=data, cfg=cfg):
         """The seven launches of rank r's step, in order, as (name, callable)."""
+        H = cfg.hidden_dim
         a, d, g = lw.ranks[r], data[r], lw.trace[r]
         T = d.num_tokens
         R = int(g["recv_counts"].sum().item())
@@ -202,7 +221,7 @@ def main():
     # kernel out of the WHOLE step does not give a usable figure: with the small exchange stand-ins in
     # the graph the parts add up to between 3 us less and 1 us more than the whole, and the sum moves
     # by microseconds between builds whose whole step differs by half a microsecond.)
-    def path_costs(stages, T, R, per_kernel=True, alone=False):
+    def path_costs(stages, T, R, per_kernel=True, alone=False, K=K, H=H):
         reps = args.kernel_reps
         path = [(n, f) for n, f in stages if n in PATH]
         chain_us = time_graph(graph_of([f for _, f in path], reps), reps)
@@ -306,6 +325,7 @@ def main():
                         f"experts_per_token={K}, hidden_dim={H}, num_tokens={T}, routing={wl['routing']}, "
                         f"weights={wl['weights']}, seed={args.seed}",
             "rows_sent": T * K, "rows_received": R, "mode": args.mode,
+            "binding": args.binding,
             "value_includes": "exchange and expert stand-ins",
         },
         "step_us_median": round(statistics.median(batches), 3),
@@ -348,22 +368,100 @@ def main():
         out["hot_path_frac_min_over_ranks"] = min(fr)
         out["hot_path_frac_mean_over_ranks"] = round(sum(fr) / len(fr), 4)
 
-    # ---- the reference's entry point: one call steps the whole job on this GPU (all ranks' kernels,
-    # W*W exchange legs per direction, two read-backs of the counts)
-    from amd_distributed_2025_amd import custom_kernel, set_peer_inputs
+    # ---- the same path on the other workload BASELINE names at this shape (C5: Zipf-skewed routing;
+    # rank 0 and the ranks that receive the most and the fewest rows, with their realised row
+    # counts) and on C4 with the reference's own input rules (fp16 tokens and `rand` weights,
+    # all2all/reference.py:16-17,37-43). One job each, set up like the main one.
+    def hot_path_of(workload, pick_ranks):
+        world_, cfg_, data_, lw_, _ = set_up(workload)
+        W_ = len(world_)
+        rows = [int(lw_.trace[r]["recv_counts"].sum().item()) for r in range(W_)]
+        res = {}
+        for r in pick_ranks(rows):
+            if str(r) in res:
+                continue
+            st_r, T_r, R_r, _ = stages_of(r, lw_, data_, cfg_)
+            hot_r, _, alg_r = path_costs(st_r, T_r, R_r, per_kernel=False, K=cfg_.experts_per_token,
+                                         H=cfg_.hidden_dim)
+            res[str(r)] = {"rows_sent": T_r * cfg_.experts_per_token, "rows_received": R_r,
+                           "hot_path_us": round(hot_r, 3), "hot_path_alg_bytes": alg_r,
+                           "frac": round(alg_r / hot_r * 1e-3 / HBM_PEAK_GBPS, 4)}
+        del lw_, data_
+        torch.cuda.empty_cache()
+        return res, rows
+
+    if args.workload == "C4" and not args.no_extra_workloads and not (args.dtype or args.weights):
+        res, rows = hot_path_of(WORKLOADS["C5"], lambda n: [0, n.index(max(n)), n.index(min(n))])
+        hot, cold = rows.index(max(rows)), rows.index(min(rows))
+        out["c5"] = {
+            "workload": f"C5: the C4 shape with routing=zipf (s=1.2), seed={args.seed}",
+            "rows_received_per_rank": rows,
+            "rank0": res["0"], "hottest_rank": hot, "hottest": res[str(hot)],
+            "coldest_rank": cold, "coldest": res[str(cold)],
+            "hot_path_frac_of_hbm_peak": res["0"]["frac"],
+        }
+        res, _ = hot_path_of(dict(WORKLOADS["C4"], dtype="fp16", weights="rand"), lambda n: [r0])
+        out["c4_fp16_rand"] = dict(res[str(r0)], workload=f"C4 with dtype=fp16, weights=rand (the reference's "
+                                   f"input rules), rank {r0}, seed={args.seed}",
+                                   hot_path_frac_of_hbm_peak=res[str(r0)]["frac"])
+
+    # ---- the reference's entry point: one call steps the whole job on this GPU (all ranks' kernels and
+    # one gathering exchange launch per rank and direction). The first call of a job runs launch by
+    # launch, the second captures it, later ones replay the capture.
+    from amd_distributed_2025_amd import HIPAllToAll, custom_kernel, custom_kernel_job, run_lockstep, set_peer_inputs
 
     world_dev = [(c, d, r, w) for (c, _, r, w), d in zip(world, data)]
     set_peer_inputs(world_dev)
-    walls = []
-    for _ in range(7):
-        torch.cuda.synchronize()
-        t1 = time.perf_counter()
-        yk = custom_kernel(world_dev[r0])
-        torch.cuda.synchronize()
-        walls.append((time.perf_counter() - t1) * 1e6)
+
+    def wall_of(fn, calls=9, skip=3):
+        walls = []
+        for _ in range(calls):
+            torch.cuda.synchronize()
+            t1 = time.perf_counter()
+            res = fn()
+            torch.cuda.synchronize()
+            walls.append((time.perf_counter() - t1) * 1e6)
+        return statistics.median(walls[skip:]), walls, res
+
+    ck_us, ck_walls, yk = wall_of(lambda: custom_kernel(world_dev[r0]))
+    job_us, _, yjob = wall_of(lambda: custom_kernel_job(world_dev))
     set_peer_inputs(None)
-    out["custom_kernel_wall_us"] = round(statistics.median(walls[2:]), 1)
-    out["custom_kernel_matches_step"] = bool(torch.equal(yk, ys0[r0]))
+    out["custom_kernel_wall_us"] = round(ck_us, 1)
+    out["custom_kernel_first_call_us"] = round(ck_walls[0], 1)
+    out["custom_kernel_job_wall_us"] = round(job_us, 1)
+    out["custom_kernel_job_wall_us_per_rank"] = round(job_us / W, 1)
+    out["custom_kernel_matches_step"] = bool(torch.equal(yk, ys0[r0]) and
+                                             all(torch.equal(a_, b_) for a_, b_ in zip(yjob, ys0)))
+
+    # ---- the reference's class surface, launch by launch: every rank of the job in a thread of its own
+    # calls dispatch() and combine() (all2all/reference.py:259-272 with the stand-in expert), through
+    # each binding; wall time of the whole job, nothing read back from the device in between
+    def class_surface(binding):
+        objs = {}
+
+        def rank_main(r, exchange):
+            a = objs.get(r)
+            if a is None:
+                a = objs[r] = HIPAllToAll(cfg, r, W, exchange=exchange, device=dev, binding=binding)
+            a.exchange = exchange  # (every job gets a new exchange object from run_lockstep)
+            d = data[r]
+            num, ex, em = a.dispatch(d.x, d.indices)
+            ey = a.expert_scale(ex, num)
+            y_ = a._buf("y_surface", (cfg.max_num_tokens, H), cfg.out_dtype)
+            y_.zero_()
+            a.combine(y_, d.weights, em, ey, num)
+            return y_[: d.num_tokens]
+
+        us, _, ys_ = wall_of(lambda: run_lockstep(W, rank_main, device=dev), calls=7, skip=2)
+        return us, bool(all(torch.equal(a_, b_) for a_, b_ in zip(ys_, ys0)))
+
+    if W > 1:
+        surf = {}
+        for b_name in ("ctypes", "ext"):
+            us, same = class_surface(b_name)
+            surf[b_name] = {"job_wall_us": round(us, 1), "per_rank_us": round(us / W, 1), "matches_step": same}
+        out["class_surface_eager"] = dict(surf, measure="dispatch() + expert stand-in + combine() of every rank, one "
+                                          "thread per rank, loose launch sizes, median wall time of 5 jobs")
 
     # ---- the expert computation a model runs between the two halves: the grouped GEMM over this
     # rank's expert-major rows (random weights; the stand-in of the reference stays in the step above)

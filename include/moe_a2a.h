@@ -401,6 +401,33 @@ int moe_a2a_exchange_local(int32_t world_size, int32_t hidden_dim,
                            int32_t rows_hint, int32_t send_capacity_rows,
                            int32_t recv_capacity_rows, void* stream);
 
+/*
+ * The same stand-in for every source of one destination rank in one launch:
+ * what the three dist.all_to_all_single calls at all2all/reference.py:88-91 and
+ * :107-119 (dispatch), :181-185 and :210-222 (combine) deliver to ONE rank.
+ *
+ *   send_bufs, send_metas, send_counts   host arrays of world_size device
+ *                 pointers: what each source rank's send half wrote
+ *                 (send_counts[s] is int32[world_size] of source s)
+ *   recv_buf, recv_meta   the destination's receive buffers; the rows of source
+ *                 s land behind the rows of the sources below it
+ *   recv_counts   int32[world_size] out: recv_counts[s] = send_counts[s][dst_rank]
+ *                 (cut to send_capacity_rows), written by the same launch
+ *   rows_hint     rows expected from one source (sizes the launch; any number
+ *                 of rows is moved)
+ *   send_capacity_rows   rows every send buffer was allocated with
+ *   recv_capacity_rows   rows the receive buffers were allocated with
+ * world_size <= 64 (MOE_A2A_EINVAL beyond: use one moe_a2a_exchange_local per
+ * leg). One launch instead of world_size launches and a copy of the counts.
+ */
+int moe_a2a_exchange_gather_local(int32_t world_size, int32_t hidden_dim,
+                                  const void* const* send_bufs,
+                                  const int32_t* const* send_metas,
+                                  const int32_t* const* send_counts, int32_t dst_rank,
+                                  void* recv_buf, int32_t* recv_meta, int32_t* recv_counts,
+                                  int32_t rows_hint, int32_t send_capacity_rows,
+                                  int32_t recv_capacity_rows, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

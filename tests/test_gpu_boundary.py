@@ -270,3 +270,124 @@ def test_oracle_expert_scale_equals_torch_on_the_device(name_in, name_out):
         nan = np.isnan(orc.b16_to_f32(want, name_out))
         assert np.array_equal(got[~nan], want[~nan]), rank
         assert np.isnan(orc.b16_to_f32(got[nan], name_out)).all(), rank
+
+
+# ----------------------------------------------------------------------------- gathering exchange
+
+@pytest.mark.parametrize("H,dt", [(72, torch.bfloat16), (2048, torch.float16), (67, torch.bfloat16)])
+def test_gathering_exchange_equals_its_legs(H, dt):
+    """`moe_a2a_exchange_gather_local` for one destination against one `moe_a2a_exchange_local` per
+    source: the same rows, meta rows and counts, including a source that holds nothing for the
+    destination, counts above the stated capacity, and rows that are not 16 bytes long."""
+    print(f"gathering exchange H={H} {dt}", flush=True)
+    from amd_distributed_2025_amd import _binding
+    import ctypes as C
+    from amd_distributed_2025_amd import _lib
+
+    W, CAP, SENT = 5, 40, -777
+    rng = np.random.default_rng(H)
+    b = _binding.get("ctypes")
+    st = torch.cuda.current_stream().cuda_stream
+    counts = rng.integers(0, 9, (W, W)).astype(np.int32)      # [src][dst]
+    counts[2, :] = 0                                           # a source with nothing to send
+    counts[3, 1] = 1000                                        # a count beyond what its buffer holds
+    bufs = [torch.from_numpy(rng.integers(0, 0x4400, (CAP, H), dtype=np.int16)).view(dt).to(DEV) for _ in range(W)]
+    metas = [torch.from_numpy(rng.integers(0, 99, (CAP, 5)).astype(np.int32)).to(DEV) for _ in range(W)]
+    cnts = [torch.from_numpy(counts[s]).to(DEV) for s in range(W)]
+    for dst in range(W):
+        for binding in ("ctypes", "ext"):
+            bb = _binding.get(binding)
+            got_buf = torch.zeros(CAP, H, dtype=dt, device=DEV)
+            got_meta = torch.full((CAP, 5), SENT, dtype=torch.int32, device=DEV)
+            got_cnt = torch.full((W,), SENT, dtype=torch.int32, device=DEV)
+            src = bb.gather_sources(H, bufs, metas, cnts)
+            for hint in (0, 3, CAP):
+                got_meta.fill_(SENT)
+                bb.exchange_gather(W, H, src, dst, got_buf, got_meta, got_cnt, hint, st)
+                want_buf = torch.zeros(CAP, H, dtype=dt, device=DEV)
+                want_meta = torch.full((CAP, 5), SENT, dtype=torch.int32, device=DEV)
+                want_cnt = torch.from_numpy(np.minimum(counts[:, dst], CAP)).to(DEV)
+                for s in range(W):
+                    b.exchange_local(W, H, bufs[s], metas[s], cnts[s], dst, want_buf, want_meta, want_cnt, s, CAP, st)
+                torch.cuda.synchronize()
+                assert torch.equal(got_cnt, want_cnt), (dst, binding, hint)
+                assert torch.equal(got_meta, want_meta), (dst, binding, hint)
+                n = int((got_meta[:, 0] != SENT).sum())
+                assert torch.equal(got_buf[:n].view(torch.int16), want_buf[:n].view(torch.int16)), (dst, binding, hint)
+    # more ranks than one launch serves, null tables
+    one = C.c_void_p(16)
+    table = (C.c_void_p * 65)(*([16] * 65))
+    lib = _lib.load()
+    assert lib.moe_a2a_exchange_gather_local(65, H, table, table, table, 0, one, one, one, 1, 4, 4, None) == -1
+    assert lib.moe_a2a_exchange_gather_local(4, H, None, table, table, 0, one, one, one, 1, 4, 4, None) == -1
+    assert lib.moe_a2a_exchange_gather_local(4, H, table, table, table, 4, one, one, one, 1, 4, 4, None) == -1
+
+
+def test_class_surface_without_counts_takes_the_short_stream_entry_points():
+    """`dispatch()` through `LocalExchange` with loose launch sizes gets no row count from the
+    exchange. The entry point is then chosen for the rows balanced routing delivers, not for the
+    capacity of the receive buffers: at C4 (2048 rows expected, 16384 rows of capacity) no planning
+    launch runs and no `row_position` workspace is made."""
+    world = generate_world(WORKLOADS["C4"], 5)
+    cfg, W = world[0][0], len(world)
+    dev = [d.to(DEV) for _, d, _, _ in world]
+    objs = {}
+
+    def rank_main(rank, exchange):
+        a = objs[rank] = HIPAllToAll(cfg, rank, W, exchange=exchange, device=DEV)
+        num, ex, em = a.dispatch(dev[rank].x, dev[rank].indices)
+        ey = a.expert_scale(ex, num)
+        y = torch.zeros(cfg.max_num_tokens, cfg.hidden_dim, dtype=cfg.out_dtype, device=DEV)
+        a.combine(y, dev[rank].weights, em, ey, num)
+        torch.cuda.synchronize()
+        return y[: dev[rank].num_tokens].clone()
+
+    ys = run_lockstep(W, rank_main, exact_hints=False, device=DEV)
+    want = run_oracle(world)
+    for r in range(W):
+        assert "row_position" not in objs[r]._ws and "entry_row" not in objs[r]._ws, r
+        assert np.array_equal(bits(ys[r]), want[r].y), r
+
+
+# ----------------------------------------------------------------------------- the entry point, call after call
+
+def test_custom_kernel_call_after_call_with_changing_inputs():
+    """The first call of a job runs launch by launch, the second captures the job, later ones replay
+    it: every call must give the oracle's bits for the inputs of THAT call, also when the inputs
+    (and with them every count the launches were sized by) change between calls, and when a job of
+    other token counts comes in between."""
+    from amd_distributed_2025_amd import custom_kernel, custom_kernel_job, set_peer_inputs
+
+    wl = dict(WORKLOADS["C3"], num_tokens="full")
+    try:
+        for call, seed in enumerate([1, 2, 3, 4]):
+            world = generate_world(wl, seed)
+            on_dev = [(c, d.to(DEV), r, w) for c, d, r, w in world]
+            want = run_oracle(world)
+            set_peer_inputs(on_dev)
+            y3 = custom_kernel(on_dev[3])
+            ys = custom_kernel_job(on_dev)
+            torch.cuda.synchronize()
+            assert np.array_equal(bits(y3), want[3].y), f"call {call}"
+            for r in range(len(world)):
+                assert np.array_equal(bits(ys[r]), want[r].y), f"call {call} rank {r}"
+            if call == 2:  # a job with other token counts in between (its own first call)
+                other = generate_world(WORKLOADS["C3"], 9)
+                other_dev = [(c, d.to(DEV), r, w) for c, d, r, w in other]
+                set_peer_inputs(other_dev)
+                yo = custom_kernel_job(other_dev)
+                torch.cuda.synchronize()
+                wo = run_oracle(other)
+                for r in range(len(other)):
+                    assert np.array_equal(bits(yo[r]), wo[r].y), f"other job rank {r}"
+        # skewed routing after uniform on the same captured job: launches sized for other counts
+        world = generate_world(dict(wl, routing="zipf"), 6)
+        on_dev = [(c, d.to(DEV), r, w) for c, d, r, w in world]
+        set_peer_inputs(on_dev)
+        ys = custom_kernel_job(on_dev)
+        torch.cuda.synchronize()
+        want = run_oracle(world)
+        for r in range(len(world)):
+            assert np.array_equal(bits(ys[r]), want[r].y), f"zipf rank {r}"
+    finally:
+        set_peer_inputs(None)
