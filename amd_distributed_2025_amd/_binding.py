@@ -103,6 +103,34 @@ class CtypesBinding:
                   rows_hint, _rows(send_buf, send_meta, hidden_dim), _rows(recv_buf, recv_meta, hidden_dim),
                   C.c_void_p(stream))
 
+    # ---- the compact expert-major layout (rows of the experts back to back)
+
+    def dispatch_recv_compact(self, shape, recv_buf, recv_meta, recv_counts, rows_hint, expert_num_tokens,
+                              expert_offsets, expert_x, expert_meta, send_back_plan, stream):
+        capacity = _rows(recv_buf, recv_meta, shape.hidden_dim)
+        _lib.call("moe_a2a_dispatch_recv_compact", C.byref(shape), _ptr(recv_buf), _ptr(recv_meta),
+                  _ptr(recv_counts), min(rows_hint, capacity), capacity, _ptr(expert_num_tokens),
+                  _ptr(expert_offsets), _ptr(expert_x), _ptr(expert_meta),
+                  _rows(expert_x, expert_meta, shape.hidden_dim), _ptr(send_back_plan), C.c_void_p(stream))
+
+    def expert_scale_compact(self, shape, expert_x, expert_num_tokens, rows_hint, expert_y, stream):
+        _lib.call("moe_a2a_expert_scale_compact", C.byref(shape), _ptr(expert_x), _ptr(expert_num_tokens),
+                  rows_hint, min(expert_x.shape[0], expert_y.shape[0]), _DT[expert_x.dtype], _DT[expert_y.dtype],
+                  _ptr(expert_y), C.c_void_p(stream))
+
+    def expert_gemm_compact(self, shape, expert_x, expert_num_tokens, rows_hint, weights, bias, expert_y, stream):
+        _lib.call("moe_a2a_expert_gemm_compact", C.byref(shape), _ptr(expert_x), _ptr(expert_num_tokens),
+                  rows_hint, min(expert_x.shape[0], expert_y.shape[0]), _ptr(weights), _ptr(bias),
+                  weights.shape[2], weights.shape[1], _DT[expert_x.dtype], _ptr(expert_y), C.c_void_p(stream))
+
+    def combine_send_compact(self, shape, expert_y, expert_meta, expert_num_tokens, rows_hint, send_buf,
+                             send_meta, send_counts, send_back_plan, stream):
+        capacity = _rows(send_buf, send_meta, shape.hidden_dim)
+        _lib.call("moe_a2a_combine_send_compact", C.byref(shape), _ptr(expert_y), _ptr(expert_meta),
+                  _ptr(expert_num_tokens), min(rows_hint, capacity),
+                  _rows(expert_y, expert_meta, shape.hidden_dim), capacity, _ptr(send_buf), _ptr(send_meta),
+                  _ptr(send_counts), _ptr(send_back_plan), C.c_void_p(stream))
+
     def gather_sources(self, hidden_dim, send_bufs, send_metas, send_counts):
         """The per-source pointer tables of `exchange_gather`, built once for buffers that stay where
         they are (a workspace): (tables, rows every send buffer holds, the tensors kept alive)."""
@@ -173,6 +201,25 @@ class ExtBinding:
                        recv_meta, recv_counts, src_rank, rows_hint, stream):
         self._m.a2a_exchange_local(world_size, hidden_dim, send_buf, send_meta, send_counts, dst_rank, recv_buf,
                                    recv_meta, recv_counts, src_rank, rows_hint, stream)
+
+    def dispatch_recv_compact(self, shape, recv_buf, recv_meta, recv_counts, rows_hint, expert_num_tokens,
+                              expert_offsets, expert_x, expert_meta, send_back_plan, stream):
+        self._m.a2a_dispatch_recv_compact(self._shape(shape), recv_buf, recv_meta, recv_counts, rows_hint,
+                                          expert_num_tokens, expert_offsets, expert_x, expert_meta,
+                                          send_back_plan, stream)
+
+    def expert_scale_compact(self, shape, expert_x, expert_num_tokens, rows_hint, expert_y, stream):
+        self._m.a2a_expert_scale_compact(self._shape(shape), expert_x, expert_num_tokens, rows_hint, expert_y,
+                                         stream)
+
+    def expert_gemm_compact(self, shape, expert_x, expert_num_tokens, rows_hint, weights, bias, expert_y, stream):
+        self._m.a2a_expert_gemm_compact(self._shape(shape), expert_x, expert_num_tokens, rows_hint, weights, bias,
+                                        expert_y, stream)
+
+    def combine_send_compact(self, shape, expert_y, expert_meta, expert_num_tokens, rows_hint, send_buf,
+                             send_meta, send_counts, send_back_plan, stream):
+        self._m.a2a_combine_send_compact(self._shape(shape), expert_y, expert_meta, expert_num_tokens, rows_hint,
+                                         send_buf, send_meta, send_counts, send_back_plan, stream)
 
     def gather_sources(self, hidden_dim, send_bufs, send_metas, send_counts):
         return (list(send_bufs), list(send_metas), list(send_counts))

@@ -51,6 +51,10 @@ SIGNATURES = {
     "moe_a2a_linear": [_P, _P, _P, _I, _I, _I, _I, _P, _P],
     "moe_a2a_exchange_local": [_I, _I, _P, _P, _P, _I, _P, _P, _P, _I, _I, _I, _I, _P],
     "moe_a2a_exchange_gather_local": [_I, _I, _P, _P, _P, _I, _P, _P, _P, _I, _I, _I, _P],
+    "moe_a2a_dispatch_recv_compact": [_SP, _P, _P, _P, _I, _I, _P, _P, _P, _P, _I, _P, _P],
+    "moe_a2a_expert_scale_compact": [_SP, _P, _P, _I, _I, _I, _I, _P, _P],
+    "moe_a2a_expert_gemm_compact": [_SP, _P, _P, _I, _I, _P, _P, _I, _I, _I, _P, _P],
+    "moe_a2a_combine_send_compact": [_SP, _P, _P, _P, _I, _I, _I, _P, _P, _P, _P, _P],
 }
 STRING_FUNCTIONS = {"moe_a2a_version": [], "moe_a2a_build_id": [], "moe_a2a_strerror": [_I]}
 

@@ -59,7 +59,8 @@ class HIPAllToAll:
     META_DIM = META_DIM  # global_exp, src_rank, src_token, src_k, pad
 
     def __init__(self, cfg: MoEConfig, rank: int, world_size: int, exchange=None, device=None,
-                 reuse_placement: bool = True, binding: str = "ctypes"):
+                 reuse_placement: bool = True, binding: str = "ctypes", layout: str = "padded",
+                 compact_rows: Optional[int] = None):
         if cfg.num_experts % world_size:
             raise ValueError("num_experts must be a multiple of world_size")
         self.cfg = cfg
@@ -78,6 +79,20 @@ class HIPAllToAll:
         # rows this rank can receive: every peer may route min(K, nle) entries of each token here
         self.max_rows_in = self.max_recv * min(cfg.experts_per_token, self.num_local_experts)
         self.max_rows_out = cfg.max_num_tokens * cfg.experts_per_token
+        # "padded": the reference's expert buffers [nle, max_recv, H] (all2all/reference.py:123-136).
+        # "compact": the experts' rows back to back in buffers of `compact_rows` rows (default: every
+        # row the rank can receive), row pos of expert le at expert_offsets[le] + pos; dispatch()
+        # then returns 2-D expert_x / expert_meta, which expert_scale, expert_gemm and combine accept.
+        if layout not in ("padded", "compact"):
+            raise ValueError(f"layout must be 'padded' or 'compact', got {layout!r}")
+        self.layout = layout
+        self.compact_rows = self.max_rows_in if compact_rows is None else int(compact_rows)
+        if layout == "compact":
+            if self.compact_rows < 1:
+                raise ValueError("compact_rows must be at least 1")
+            # a rank that keeps at most compact_rows rows needs no room to receive or return more
+            self.max_rows_in = min(self.max_rows_in, self.compact_rows)
+        self.expert_offsets = None  # compact layout: int32[nle + 1], written by dispatch_recv
         self._ws = {}
         # dispatch_recv leaves a plan of where combine_send will put every row; combine_send uses
         # it when it is handed the very tensors that dispatch_recv returned
@@ -93,6 +108,10 @@ class HIPAllToAll:
             t = torch.empty(tuple(shape), dtype=dtype, device=self.device)
             self._ws[name] = t
         return t
+
+    def workspace_bytes(self) -> int:
+        """Device memory of the buffers this object has made so far."""
+        return sum(t.numel() * t.element_size() for t in self._ws.values())
 
     def inbound_buffers(self, phase: str):
         """Where an exchange should deliver this rank's incoming rows.
@@ -165,12 +184,19 @@ class HIPAllToAll:
         hint = min(capacity, self.max_rows_out if rows_hint is None else int(rows_hint))
         nle = self.num_local_experts
         num = self._buf("expert_num_tokens", (nle,), torch.int32)
-        ex = self._buf("expert_x", (nle, self.max_recv, cfg.hidden_dim), cfg.in_dtype)
-        em = self._buf("expert_meta", (nle, self.max_recv, META_DIM), torch.int32)
         plan = self._buf("send_back_plan", (2 * cfg.num_experts,), torch.int32) if self.reuse_placement else None
-        pos = self._buf("row_position", (capacity,), torch.int32) if hint > self._long_from("dispatch") else None
-        self.binding.dispatch_recv(self.shape, recv_buf, recv_meta, recv_counts, hint, num, ex, em, plan,
-                                   _stream(self.device), pos)
+        if self.layout == "compact":
+            ex = self._buf("expert_x", (self.compact_rows, cfg.hidden_dim), cfg.in_dtype)
+            em = self._buf("expert_meta", (self.compact_rows, META_DIM), torch.int32)
+            self.expert_offsets = self._buf("expert_offsets", (nle + 1,), torch.int32)
+            self.binding.dispatch_recv_compact(self.shape, recv_buf, recv_meta, recv_counts, hint, num,
+                                               self.expert_offsets, ex, em, plan, _stream(self.device))
+        else:
+            ex = self._buf("expert_x", (nle, self.max_recv, cfg.hidden_dim), cfg.in_dtype)
+            em = self._buf("expert_meta", (nle, self.max_recv, META_DIM), torch.int32)
+            pos = self._buf("row_position", (capacity,), torch.int32) if hint > self._long_from("dispatch") else None
+            self.binding.dispatch_recv(self.shape, recv_buf, recv_meta, recv_counts, hint, num, ex, em, plan,
+                                       _stream(self.device), pos)
         self._planned_for = None if plan is None else (em.data_ptr(), num.data_ptr())
         self._rows_in_hint = hint
         return num, ex, em
@@ -182,7 +208,10 @@ class HIPAllToAll:
         _need(expert_num_tokens, torch.int32, self.device, "expert_num_tokens")
         hint = self._default_rows_in(rows_hint)
         ey = self._buf("expert_y", tuple(expert_x.shape), cfg.out_dtype)
-        self.binding.expert_scale(self.shape, expert_x, expert_num_tokens, hint, ey, _stream(self.device))
+        if expert_x.dim() == 2:  # the compact layout
+            self.binding.expert_scale_compact(self.shape, expert_x, expert_num_tokens, hint, ey, _stream(self.device))
+        else:
+            self.binding.expert_scale(self.shape, expert_x, expert_num_tokens, hint, ey, _stream(self.device))
         return ey
 
     def expert_gemm(self, expert_x, expert_num_tokens, weights, bias=None, rows_hint: Optional[int] = None,
@@ -204,9 +233,12 @@ class HIPAllToAll:
         _need(expert_x, dt, self.device, "expert_x")
         _need(expert_num_tokens, torch.int32, self.device, "expert_num_tokens")
         _need(weights, dt, self.device, "weights")
-        if expert_x.dim() != 3 or tuple(expert_x.shape[:2]) != (nle, self.max_recv):
-            raise ValueError(f"expert_x must be [{nle}, {self.max_recv}, in_dim], got {tuple(expert_x.shape)}")
-        in_dim = expert_x.shape[2]
+        compact = expert_x.dim() == 2  # [rows, in_dim]: the experts' rows back to back
+        if not compact and (expert_x.dim() != 3 or tuple(expert_x.shape[:2]) != (nle, self.max_recv)):
+            raise ValueError(f"expert_x must be [{nle}, {self.max_recv}, in_dim] or [rows, in_dim], "
+                             f"got {tuple(expert_x.shape)}")
+        in_dim = expert_x.shape[-1]
+        rows_shape = tuple(expert_x.shape[:-1])
         if weights.dim() != 3 or weights.shape[0] != nle or weights.shape[2] != in_dim:
             raise ValueError(f"weights must be [{nle}, out_dim, {in_dim}], got {tuple(weights.shape)}")
         out_dim = weights.shape[1]
@@ -219,13 +251,13 @@ class HIPAllToAll:
             name = f"expert_out_{out_dim}"
             if name in self._ws and self._ws[name].data_ptr() == expert_x.data_ptr():
                 name += "_b"  # a layer of equal width reading the buffer the one before it wrote
-            out = self._buf(name, (nle, self.max_recv, out_dim), dt)
+            out = self._buf(name, rows_shape + (out_dim,), dt)
         else:
             _need(out, dt, self.device, "out")
-            if tuple(out.shape) != (nle, self.max_recv, out_dim) or out.data_ptr() == expert_x.data_ptr():
-                raise ValueError(f"out must be [{nle}, {self.max_recv}, {out_dim}] and not the input")
-        self.binding.expert_gemm(self.shape, expert_x, expert_num_tokens, hint, weights, bias, out,
-                                 _stream(self.device))
+            if tuple(out.shape) != rows_shape + (out_dim,) or out.data_ptr() == expert_x.data_ptr():
+                raise ValueError(f"out must be {list(rows_shape) + [out_dim]} and not the input")
+        gemm = self.binding.expert_gemm_compact if compact else self.binding.expert_gemm
+        gemm(self.shape, expert_x, expert_num_tokens, hint, weights, bias, out, _stream(self.device))
         return out
 
     def combine_send(self, expert_meta, expert_y, expert_num_tokens, rows_hint: Optional[int] = None):
@@ -236,7 +268,11 @@ class HIPAllToAll:
         _need(expert_meta, torch.int32, self.device, "expert_meta")
         _need(expert_y, cfg.out_dtype, self.device, "expert_y")
         _need(expert_num_tokens, torch.int32, self.device, "expert_num_tokens")
-        if tuple(expert_y.shape) != (self.num_local_experts, self.max_recv, cfg.hidden_dim):
+        compact = expert_y.dim() == 2
+        if compact:
+            if expert_y.shape[1] != cfg.hidden_dim or expert_meta.dim() != 2:
+                raise ValueError("combine: compact expert_y / expert_meta must be [rows, hidden_dim] / [rows, 5]")
+        elif tuple(expert_y.shape) != (self.num_local_experts, self.max_recv, cfg.hidden_dim):
             raise ValueError("combine: expert_y must be [num_local_experts, max_recv, hidden_dim]")
         hint = self._default_rows_in(rows_hint)
         counts = self._buf("back_counts", (self.world_size,), torch.int32)
@@ -248,8 +284,9 @@ class HIPAllToAll:
         plan = None
         if self._planned_for == (expert_meta.data_ptr(), expert_num_tokens.data_ptr()):
             plan = self._ws["send_back_plan"]
-        self.binding.combine_send(self.shape, expert_y, expert_meta, expert_num_tokens,
-                                  min(hint, self.max_rows_in), buf, meta, counts, plan, _stream(self.device))
+        send = self.binding.combine_send_compact if compact else self.binding.combine_send
+        send(self.shape, expert_y, expert_meta, expert_num_tokens, min(hint, self.max_rows_in), buf, meta, counts,
+             plan, _stream(self.device))
         return counts, buf, meta
 
     def combine_recv(self, out_tokens, weights, ret_counts, ret_buf, ret_meta, accumulate: bool = True):
@@ -417,10 +454,12 @@ class LocalWorld:
 
     def __init__(self, cfg: MoEConfig, world_size: int, device=None, exact_hints: bool = True,
                  reuse_placement: bool = True, binding: str = "ctypes",
-                 long_stream_rows: Optional[int] = None):
+                 long_stream_rows: Optional[int] = None, layout: str = "padded",
+                 compact_rows: Optional[int] = None):
         self.cfg, self.world_size = cfg, world_size
         self.ranks = [HIPAllToAll(cfg, r, world_size, device=device, reuse_placement=reuse_placement,
-                                  binding=binding) for r in range(world_size)]
+                                  binding=binding, layout=layout, compact_rows=compact_rows)
+                      for r in range(world_size)]
         if long_stream_rows is not None:  # (0: every receive half takes the long-stream entry points)
             for a in self.ranks:
                 a.long_stream_rows = long_stream_rows

@@ -29,7 +29,8 @@ EXT_NAME = "moe_a2a_torch"
 # the wrappers load_inline binds, one per entry point of the C ABI
 EXT_FUNCTIONS = ["a2a_version", "a2a_dispatch_send", "a2a_plan_send", "a2a_dispatch_recv", "a2a_combine_send",
                  "a2a_combine_recv", "a2a_expert_scale", "a2a_expert_gemm", "a2a_linear", "a2a_exchange_local",
-                 "a2a_exchange_gather_local"]
+                 "a2a_exchange_gather_local", "a2a_dispatch_recv_compact", "a2a_expert_scale_compact",
+                 "a2a_expert_gemm_compact", "a2a_combine_send_compact"]
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950",

@@ -917,15 +917,26 @@ __global__ __launch_bounds__(RPLAN_BLOCK) void plan_recv_kernel(
   }
 }
 
-// POS: the position of every row inside its expert comes from `row_pos` (plan_recv_kernel);
-// the movers scan nothing.
-template <typename V, int NVW, bool PLAN, bool POS>
+// How a mover finds the place of a row:
+//   RECV_SCAN     by counting the earlier rows of the same expert (the padded layout of
+//                 all2all/reference.py:127-136: row pos of expert le at le * max_recv + pos);
+//   RECV_POS      from `row_pos` (plan_recv_kernel): the movers scan nothing (padded layout);
+//   RECV_COMPACT  the compact layout: the experts' rows back to back, row pos of expert le at
+//                 offset[le] + pos with offset = exclusive prefix of the rows per expert. A row's
+//                 place is then the number of rows of lower experts anywhere in the stream plus
+//                 the earlier rows of its own expert (one pass over all keys); `max_recv` is the
+//                 number of rows the compact buffers hold, and the counting workgroups also write
+//                 the offsets.
+enum { RECV_SCAN = 0, RECV_POS = 1, RECV_COMPACT = 2 };
+
+template <typename V, int NVW, bool PLAN, int MODE>
 __global__ __launch_bounds__(64 * ROWS) void dispatch_recv_kernel(
     const V* __restrict__ recv_buf, const int* __restrict__ recv_meta,
     const int* __restrict__ recv_counts, int W, int hint_rows, int capacity_rows, int nle,
     uint32_t magic, int max_recv, int row_vecs, int chunks, int* __restrict__ expert_num_tokens,
     V* __restrict__ expert_x, int* __restrict__ expert_meta, int* __restrict__ plan,
-    const int* __restrict__ row_pos) {
+    const int* __restrict__ row_pos, int* __restrict__ expert_offsets) {
+  constexpr bool POS = MODE == RECV_POS, COMPACT = MODE == RECV_COMPACT;
   __shared__ int part[2 * ROWS * ROWS];
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const StridedKeys key{recv_meta, META};
@@ -972,6 +983,13 @@ __global__ __launch_bounds__(64 * ROWS) void dispatch_recv_kernel(
           out[1] = (incl - mine) + below;
         }
         if (lane == 63) expert_num_tokens[me] = upto;
+        if constexpr (COMPACT) {  // rows of lower experts, from every source: where this expert's rows start
+          const int lower = wave_sum(below), mine_all = __builtin_amdgcn_readlane(upto, 63);
+          if (lane == 0) {
+            expert_offsets[me] = lower;
+            if (me == nle - 1) expert_offsets[nle] = lower + mine_all;
+          }
+        }
       }
       return;
     }
@@ -983,6 +1001,14 @@ __global__ __launch_bounds__(64 * ROWS) void dispatch_recv_kernel(
     int c = count_keys<64 * ROWS>(R, key, [=](int e, int) { return floormod(e, nle, magic) == me; });
     c = block_sum<ROWS>(c, part);
     if (tid == 0) expert_num_tokens[me] = c;
+    if constexpr (COMPACT) {
+      int lower = count_keys<64 * ROWS>(R, key, [=](int e, int) { return floormod(e, nle, magic) < me; });
+      lower = block_sum<ROWS>(lower, part);
+      if (tid == 0) {
+        expert_offsets[me] = lower;
+        if (me == nle - 1) expert_offsets[nle] = lower + c;
+      }
+    }
     return;
   }
 
@@ -1017,8 +1043,9 @@ __global__ __launch_bounds__(64 * ROWS) void dispatch_recv_kernel(
     for (int r = 0; r < ROWS; ++r) re[r] = recv_meta[(size_t)min(i0 + r, limit - 1) * META];
     int m = 0;
     if (c == 0 && lane < META) m = recv_meta[(size_t)ic * META + lane];
-    // only rows before the group's last row can precede any of its rows
-    RowsScan<StridedKeys> scan(min(i0 + ROWS - 1, limit), key);
+    // only rows before the group's last row can precede any of its rows in its expert; the rows of
+    // lower experts, which the compact layout puts ahead of it, lie anywhere in the stream
+    RowsScan<StridedKeys> scan(COMPACT ? limit : min(i0 + ROWS - 1, limit), key);
     WavePayload<V, NVW> p;
     p.load(recv_buf + (size_t)ic * row_vecs, base, row_vecs, lane);
 
@@ -1027,8 +1054,10 @@ __global__ __launch_bounds__(64 * ROWS) void dispatch_recv_kernel(
 #pragma unroll
     for (int r = 0; r < ROWS; ++r) rle[r] = floormod(re[r], nle, magic);
     int cnt[ROWS];
-    scan.finish(key, min(i0 + ROWS - 1, R), [&](int r, int e2, int i2) {
-      return (floormod(e2, nle, magic) == rle[r]) & (i2 < i0 + r);
+    scan.finish(key, COMPACT ? R : min(i0 + ROWS - 1, R), [&](int r, int e2, int i2) {
+      const int le2 = floormod(e2, nle, magic);
+      if constexpr (COMPACT) return (le2 < rle[r]) | ((le2 == rle[r]) & (i2 < i0 + r));
+      else return (le2 == rle[r]) & (i2 < i0 + r);
     }, cnt);
     const int pos = rows_reduce(cnt, part, parity++, wave, lane);
 
@@ -1036,7 +1065,7 @@ __global__ __launch_bounds__(64 * ROWS) void dispatch_recv_kernel(
       int le = 0;
 #pragma unroll
       for (int r = 0; r < ROWS; ++r) le = r == wave ? rle[r] : le;
-      const size_t row = (size_t)le * max_recv + pos;
+      const size_t row = COMPACT ? (size_t)pos : (size_t)le * max_recv + pos;
       p.template store<(MOE_A2A_NT_RECV != 0)>(expert_x + row * row_vecs, base, row_vecs, lane);
       if (c == 0 && lane < META) expert_meta[row * META + lane] = m;
     }
@@ -1132,7 +1161,13 @@ struct ExpertStreamKeys {
   const int* pre;  // LDS, nle + 1 entries, pre[nle] = number of rows
   const int* __restrict__ meta;
   int nle, top, max_recv;
+  bool compact;  // the experts' rows lie back to back: stream row g is buffer row g
   __device__ __forceinline__ void fetch(const int* g, int* key) const {
+    if (compact) {
+#pragma unroll
+      for (int u = 0; u < SCAN_UNROLL; ++u) key[u] = meta[(size_t)g[u] * META + FIELD];
+      return;
+    }
     int le[SCAN_UNROLL];
 #pragma unroll
     for (int u = 0; u < SCAN_UNROLL; ++u) le[u] = 0;
@@ -1183,7 +1218,13 @@ struct WaveStreamKeys {
   int excl;  // this lane's WaveExpertPrefix::excl
   const int* __restrict__ meta;
   int nle, top, max_recv;
+  bool compact;  // the experts' rows lie back to back: stream row g is buffer row g
   __device__ __forceinline__ void fetch(const int* g, int* key) const {
+    if (compact) {  // (the same for every lane: no lane leaves the shuffles below behind)
+#pragma unroll
+      for (int u = 0; u < SCAN_UNROLL; ++u) key[u] = meta[(size_t)g[u] * META + FIELD];
+      return;
+    }
     int le[SCAN_UNROLL];
 #pragma unroll
     for (int u = 0; u < SCAN_UNROLL; ++u) le[u] = 0;
@@ -1228,18 +1269,22 @@ __global__ __launch_bounds__(64 * ROWS) void combine_send_kernel(
     const V* __restrict__ expert_y, const int* __restrict__ expert_meta,
     const int* __restrict__ expert_num_tokens, int nle, int max_recv, int W, int row_vecs,
     int chunks, int capacity_rows, V* __restrict__ send_buf, int* __restrict__ send_meta,
-    int* __restrict__ send_counts, const int* __restrict__ plan) {
+    int* __restrict__ send_counts, const int* __restrict__ plan, int compact_rows) {
   static_assert(!PLAN || SMALL, "the planned path keeps the expert prefix in registers");
   __shared__ int part[2 * ROWS * ROWS];
   __shared__ int pre[SMALL ? 1 : MAX_LOCAL_EXPERTS + 1];
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  // compact_rows > 0: expert_y / expert_meta hold the experts' rows back to back (stream row g is
+  // buffer row g) in buffers of compact_rows rows, and max_recv is that number too
+  const bool compact = compact_rows > 0;
 
   if constexpr (PLAN) {
     const int raw = lane < nle ? expert_num_tokens[lane] : 0;
-    if (__ballot(raw > max_recv) == 0) {
-      const int have = max(raw, 0);
-      const int incl = wave_inclusive_scan(have), excl = incl - have;
-      const int R = __builtin_amdgcn_readlane(incl, 63);
+    const int have = max(raw, 0);
+    const int incl = wave_inclusive_scan(have), excl = incl - have;
+    const int R = __builtin_amdgcn_readlane(incl, 63);
+    // (the plan also counts rows that found no room; with such rows the scan below is taken)
+    if (__ballot(raw > max_recv) == 0 && !(compact && R > compact_rows)) {
 
       if ((int)blockIdx.x < W) {
         // rows that go back to origin `me`: the lengths of its runs, one expert per lane
@@ -1261,7 +1306,7 @@ __global__ __launch_bounds__(64 * ROWS) void combine_send_kernel(
         const int base = c * (64 * NVW);
         const int le = __popcll(__ballot(incl <= g));
         const int j = g - __builtin_amdgcn_readlane(excl, le);
-        const size_t row = (size_t)le * max_recv + j;
+        const size_t row = compact ? (size_t)g : (size_t)le * max_recv + j;
         int run[PLAN_INTS] = {INT_MAX, 0};
         if (lane < W) __builtin_memcpy(run, plan + ((size_t)le * W + lane) * PLAN_INTS, sizeof(run));
         int m = 0;
@@ -1292,11 +1337,13 @@ __global__ __launch_bounds__(64 * ROWS) void combine_send_kernel(
   } else {
     R = expert_prefix<ROWS>(expert_num_tokens, nle, max_recv, pre, part);
   }
+  if (compact) R = min(R, compact_rows);
   Keys key;
-  if constexpr (SMALL) key = Keys{my_excl, expert_meta, nle, 32, max_recv};
-  else key = Keys{pre, expert_meta, nle, top_step(nle), max_recv};
-  // padded row index of stream row g (wave-uniform g < R)
+  if constexpr (SMALL) key = Keys{my_excl, expert_meta, nle, 32, max_recv, compact};
+  else key = Keys{pre, expert_meta, nle, top_step(nle), max_recv, compact};
+  // buffer row of stream row g (wave-uniform g < R)
   auto padded_row = [&](int g) -> size_t {
+    if (compact) return (size_t)g;
     int le, first;
     if constexpr (SMALL) {
       le = __popcll(__ballot(my_incl <= g));
@@ -1680,17 +1727,19 @@ __global__ __launch_bounds__(BLK) void combine_recv_kernel(
 template <typename V, int NV, int DIN, int DOUT>
 __global__ __launch_bounds__(BLOCK) void expert_scale_kernel(
     const V* __restrict__ expert_x, const int* __restrict__ expert_num_tokens, int nle,
-    int max_recv, float scale, int row_vecs, int chunks, V* __restrict__ expert_y) {
+    int max_recv, float scale, int row_vecs, int chunks, V* __restrict__ expert_y, int compact_rows) {
   __shared__ int red[NWAVES];
   __shared__ int pre[MAX_LOCAL_EXPERTS + 1];
-  const int R = expert_prefix<NWAVES>(expert_num_tokens, nle, max_recv, pre, red);
+  // compact_rows > 0: the experts' rows lie back to back in buffers of that many rows (= max_recv)
+  int R = expert_prefix<NWAVES>(expert_num_tokens, nle, max_recv, pre, red);
+  if (compact_rows > 0) R = min(R, compact_rows);
   const int top = top_step(nle);
   const int items = R * chunks;
   for (int q = blockIdx.x; q < items; q += gridDim.x) {
     const int g = chunks == 1 ? q : q / chunks, c = q - g * chunks;
     const int base = c * (BLOCK * NV);
-    const int le = expert_of(pre, nle, top, g);
-    const size_t row = (size_t)le * max_recv + (g - pre[le]);
+    const int le = compact_rows > 0 ? 0 : expert_of(pre, nle, top, g);
+    const size_t row = compact_rows > 0 ? (size_t)g : (size_t)le * max_recv + (g - pre[le]);
     Payload<V, NV> p;
     p.load(expert_x + row * row_vecs, base, row_vecs);
     p.map([scale](V v) {
@@ -1716,16 +1765,17 @@ __global__ __launch_bounds__(BLOCK) void expert_scale_kernel(
 template <int NVW, int DIN, int DOUT>
 __global__ __launch_bounds__(64 * ROWS) void expert_scale_wave_kernel(
     const b128* __restrict__ expert_x, const int* __restrict__ expert_num_tokens, int nle,
-    int max_recv, float scale, int row_vecs, int chunks, b128* __restrict__ expert_y) {
+    int max_recv, float scale, int row_vecs, int chunks, b128* __restrict__ expert_y, int compact_rows) {
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const WaveExpertPrefix wp(expert_num_tokens, nle, max_recv);
-  const int items = wp.total * chunks, waves = gridDim.x * ROWS;
+  const int R = compact_rows > 0 ? min(wp.total, compact_rows) : wp.total;
+  const int items = R * chunks, waves = gridDim.x * ROWS;
   for (int q = blockIdx.x * ROWS + wave; q < items; q += waves) {
     const int g = chunks == 1 ? q : q / chunks, c = q - g * chunks;
     const int base = c * (64 * NVW);
     int le, first;
     wp.locate(g, le, first);
-    const size_t row = (size_t)le * max_recv + (g - first);
+    const size_t row = compact_rows > 0 ? (size_t)g : (size_t)le * max_recv + (g - first);
     WavePayload<b128, NVW> p;
     p.load(expert_x + row * row_vecs, base, row_vecs, lane);
 #pragma unroll
@@ -1827,7 +1877,7 @@ template <int DT, int TJ, int GW>
 __global__ __launch_bounds__(64 * GW, GW > 4 ? 1 : TJ <= 2 ? MOE_A2A_GEMM_OCC : MOE_A2A_GEMM_OCC4) void expert_gemm_kernel(
     const b128* __restrict__ expert_x, const int* __restrict__ expert_num_tokens,
     const b128* __restrict__ weights, const uint16_t* __restrict__ bias, uint16_t* __restrict__ expert_y,
-    int nle, int max_recv, int N, int K, int col_tiles) {
+    int nle, int max_recv, int N, int K, int col_tiles, int compact) {
   constexpr int TOK = TJ * 32;               // tokens per block
   constexpr int D = TJ >= 4 ? MOE_A2A_GEMM_DEPTH4 : GEMM_DEPTH;
   __shared__ b128 xs[D][TOK * 8];            // D steps of TOK tokens x 8 vectors
@@ -1838,8 +1888,8 @@ __global__ __launch_bounds__(64 * GW, GW > 4 ? 1 : TJ <= 2 ? MOE_A2A_GEMM_OCC : 
   constexpr int XL = TOK * 8 / LOADERS;       // token loads of a loading lane per step (LOADERS / 8 rows each)
   static_assert(XL >= 1 && XL * LOADERS == TOK * 8 && LOADERS <= THREADS, "whole loads");
   __shared__ b128 ws[GW][32 * 8];            // per wave: one step of its 32 weight rows x 8 vectors
-  __shared__ int red[GW];
-  __shared__ int home[2];
+  __shared__ int red[GW], red_rows[GW];
+  __shared__ int home[4];
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const int row_vecs = K / 8, steps = (K + GEMM_KSTEP - 1) / GEMM_KSTEP;
   const int tail_vecs = row_vecs - (steps - 1) * 8;  // vectors of a row in the last step, 1..8
@@ -1847,11 +1897,31 @@ __global__ __launch_bounds__(64 * GW, GW > 4 ? 1 : TJ <= 2 ? MOE_A2A_GEMM_OCC : 
 
   // Blocks of tokens per expert, summed over the run of experts this thread owns and scanned over
   // the workgroup: block number g of the launch belongs to the thread with begin <= g < begin + mine.
-  auto blocks_of = [=](int le) { return (rows_of(le) + TOK - 1) / TOK; };
   const int per = (nle + THREADS - 1) / THREADS;
   const int run_b = min(tid * per, nle), run_e = min(run_b + per, nle);
+  // compact: x and y hold the experts' rows back to back in buffers of max_recv rows. The rows
+  // ahead of an expert are a prefix over the counts, and an expert only has the rows that still
+  // fit the buffers (counts that add up to more never send a load or a store past their end).
+  int mine_rows = 0;
+  for (int le = run_b; le < run_e; ++le) mine_rows += rows_of(le);
+  int rows_begin;
+  {
+    const int inc_rows = wave_inclusive_scan(mine_rows);
+    if (lane == 63) red_rows[wave] = inc_rows;
+    lds_barrier();
+    int off_rows = 0;
+#pragma unroll
+    for (int w = 0; w < GW; ++w) off_rows += w < wave ? red_rows[w] : 0;
+    rows_begin = off_rows + inc_rows - mine_rows;
+  }
+  // rows of expert le that are there: all of them in the padded layout
+  auto kept_of = [=](int le, int ahead) {
+    const int n = rows_of(le);
+    return compact ? min(ahead + n, max_recv) - min(ahead, max_recv) : n;
+  };
+  auto blocks_for = [=](int rows) { return (rows + TOK - 1) / TOK; };
   int mine = 0;
-  for (int le = run_b; le < run_e; ++le) mine += blocks_of(le);
+  for (int le = run_b, ahead = rows_begin; le < run_e; ahead += rows_of(le), ++le) mine += blocks_for(kept_of(le, ahead));
   int begin, row_blocks;
   {
     const int inc = wave_inclusive_scan(mine);
@@ -1877,20 +1947,25 @@ __global__ __launch_bounds__(64 * GW, GW > 4 ? 1 : TJ <= 2 ? MOE_A2A_GEMM_OCC : 
   for (int tile = blockIdx.x; tile < tiles; tile += stride) {
     const int rb = tile / col_tiles, ct = tile - rb * col_tiles;
     if (begin <= rb && rb < begin + mine) {  // one thread: walk its run to the expert of block rb
-      int le = run_b, first = begin;
+      int le = run_b, first = begin, rows_ahead = rows_begin;
       for (;; ++le) {
-        const int n = blocks_of(le);
+        const int n = blocks_for(kept_of(le, rows_ahead));
         if (rb < first + n) break;
         first += n;
+        rows_ahead += rows_of(le);
       }
       home[0] = le;
       home[1] = first;
+      home[2] = min(rows_ahead, max_recv);
+      home[3] = kept_of(le, rows_ahead);
     }
     lds_barrier();  // (the next write to `home` comes after the barriers of the steps below)
     // (uniform values are pinned to scalar registers: the bases below then cost no vector registers)
     const int le = __builtin_amdgcn_readfirstlane(home[0]);
-    const int rows = __builtin_amdgcn_readfirstlane(rows_of(le));
+    const int rows = __builtin_amdgcn_readfirstlane(home[3]);
     const int t0 = (rb - __builtin_amdgcn_readfirstlane(home[1])) * TOK;  // first token of the block (t0 < rows)
+    // buffer row of the expert's first row
+    const size_t row0 = compact ? (size_t)__builtin_amdgcn_readfirstlane(home[2]) : (size_t)le * max_recv;
     const int n0 = ct * (GW * 32) + __builtin_amdgcn_readfirstlane(wave) * 32;  // first output column of this wave
     const bool cols_valid = n0 < N;                      // the last tile of columns may be partly empty
     const int nw = min(n0, N - 32);                      // (a wave without columns reads valid memory)
@@ -1907,7 +1982,7 @@ __global__ __launch_bounds__(64 * GW, GW > 4 ? 1 : TJ <= 2 ? MOE_A2A_GEMM_OCC : 
     const __amdgpu_buffer_rsrc_t wbuf = __builtin_amdgcn_make_buffer_rsrc(
         (void*)(weights + ((size_t)le * N + nw) * row_vecs), 0, 32 * row_bytes, BUFFER_RAW_32BIT);
     const __amdgpu_buffer_rsrc_t xbuf = __builtin_amdgcn_make_buffer_rsrc(
-        (void*)(expert_x + ((size_t)le * max_recv + t0) * row_vecs), 0, min(live, TOK) * row_bytes, BUFFER_RAW_32BIT);
+        (void*)(expert_x + (row0 + t0) * row_vecs), 0, min(live, TOK) * row_bytes, BUFFER_RAW_32BIT);
     constexpr int OUT_OF_RANGE = 0x40000000;
     int woff[4], wslot[4], xoff[XL], wpast[2];
 #pragma unroll
@@ -2007,7 +2082,7 @@ __global__ __launch_bounds__(64 * GW, GW > 4 ? 1 : TJ <= 2 ? MOE_A2A_GEMM_OCC : 
       for (int j = 0; j < TJ; ++j) {
         const int token = t0 + j * 32 + r;
         if (token < rows) {
-          uint16_t* out = expert_y + ((size_t)le * max_recv + token) * N + n0 + kb * 4;
+          uint16_t* out = expert_y + (row0 + token) * N + n0 + kb * 4;
 #pragma unroll
           for (int g = 0; g < 4; ++g) {
             const f32x16& c = acc[j];
@@ -2181,7 +2256,7 @@ template <int DT, int WM, int WN, int TM, int TN, bool GROUPED>
 __global__ __launch_bounds__(64 * WM * WN, TM * TN >= 16 ? 1 : 2) void dense_gemm_kernel(
     const b128* __restrict__ A, const b128* __restrict__ B, const uint16_t* __restrict__ bias,
     uint16_t* __restrict__ C, int M, int N, int K, int tiles_m, int tiles_n,
-    const int* __restrict__ rows_of_group, int groups, int max_rows) {
+    const int* __restrict__ rows_of_group, int groups, int max_rows, int compact) {
   constexpr int NT = 64 * WM * WN, BM = WM * TM * 32, BN = WN * TN * 32;
   constexpr int LA = BM * 8 / NT, LB = BN * 8 / NT;  // 16-byte vectors a thread copies per step
   constexpr int GROUP_M = 4;
@@ -2197,16 +2272,33 @@ __global__ __launch_bounds__(64 * WM * WN, TM * TN >= 16 ? 1 : 2) void dense_gem
   // tiles of a run of groups, a scan over the workgroup places the runs, and the thread whose run
   // holds a row tile walks it to find the group. The launch strides over (row tile, column tile)
   // pairs, column tile fastest, so its size is a matter of speed only.
-  __shared__ int grp_red[NT / 64];
-  __shared__ int grp_home[2];
+  __shared__ int grp_red[NT / 64], grp_red_rows[NT / 64];
+  __shared__ int grp_home[4];
   [[maybe_unused]] auto rows_of = [=](int g) { return min(max(rows_of_group[g], 0), max_rows); };
-  [[maybe_unused]] auto row_tiles_of = [=](int g) { return (rows_of(g) + BM - 1) / BM; };
-  [[maybe_unused]] int run_first = 0, run_begin = 0, run_tiles = 0, total_tiles = 0;
+  // compact: A and C hold the groups' rows back to back in buffers of max_rows rows. The rows
+  // ahead of a group are a prefix over the counts, and a group only has the rows that still fit
+  // the buffers (counts that add up to more never send a load or a store past their end).
+  [[maybe_unused]] auto kept_of = [=](int g, int ahead) {
+    const int n = rows_of(g);
+    return compact ? min(ahead + n, max_rows) - min(ahead, max_rows) : n;
+  };
+  [[maybe_unused]] auto tiles_for = [=](int rows) { return (rows + BM - 1) / BM; };
+  [[maybe_unused]] int run_first = 0, run_end = 0, run_begin = 0, run_tiles = 0, total_tiles = 0, run_rows_begin = 0;
   if constexpr (GROUPED) {
     const int per = (groups + NT - 1) / NT;
     run_first = min(tid * per, groups);
-    const int run_end = min(run_first + per, groups);
-    for (int g = run_first; g < run_end; ++g) run_tiles += row_tiles_of(g);
+    run_end = min(run_first + per, groups);
+    int run_rows = 0;
+    for (int g = run_first; g < run_end; ++g) run_rows += rows_of(g);
+    const int inc_rows = wave_inclusive_scan(run_rows);
+    if (lane == 63) grp_red_rows[wave] = inc_rows;
+    lds_barrier();
+    int off_rows = 0;
+#pragma unroll
+    for (int w = 0; w < NT / 64; ++w) off_rows += w < wave ? grp_red_rows[w] : 0;
+    run_rows_begin = off_rows + inc_rows - run_rows;
+    for (int g = run_first, ahead = run_rows_begin; g < run_end; ahead += rows_of(g), ++g)
+      run_tiles += tiles_for(kept_of(g, ahead));
     const int inc = wave_inclusive_scan(run_tiles);
     if (lane == 63) grp_red[wave] = inc;
     lds_barrier();
@@ -2237,23 +2329,27 @@ __global__ __launch_bounds__(64 * WM * WN, TM * TN >= 16 ? 1 : 2) void dense_gem
     const int rb = logical / tiles_n, tn = logical - rb * tiles_n;
     lds_barrier();  // the tile before is out of LDS, and its grp_home has been read
     if (run_begin <= rb && rb < run_begin + run_tiles) {
-      int g = run_first, first = run_begin;
+      int g = run_first, first = run_begin, rows_ahead = run_rows_begin;
       for (;; ++g) {
-        const int n = row_tiles_of(g);
+        const int n = tiles_for(kept_of(g, rows_ahead));
         if (rb < first + n) break;
         first += n;
+        rows_ahead += rows_of(g);
       }
       grp_home[0] = g;
       grp_home[1] = first;
+      grp_home[2] = min(rows_ahead, max_rows);
+      grp_home[3] = kept_of(g, rows_ahead);
     }
     lds_barrier();
     const int g = __builtin_amdgcn_readfirstlane(grp_home[0]);
     const int t0 = (rb - __builtin_amdgcn_readfirstlane(grp_home[1])) * BM;
+    const size_t row0 = compact ? (size_t)__builtin_amdgcn_readfirstlane(grp_home[2]) : (size_t)g * max_rows;
     n0 = tn * BN;
-    rows_left = __builtin_amdgcn_readfirstlane(rows_of(g)) - t0;
-    a_tile = A + ((size_t)g * max_rows + t0) * row_vecs;
+    rows_left = __builtin_amdgcn_readfirstlane(grp_home[3]) - t0;
+    a_tile = A + (row0 + t0) * row_vecs;
     b_tile = B + ((size_t)g * N + n0) * row_vecs;
-    c_tile = C + ((size_t)g * max_rows + t0) * N;
+    c_tile = C + (row0 + t0) * N;
     bias_row = bias ? bias + (size_t)g * N : nullptr;
   } else {
     const int logical = xcd_contiguous(blockIdx.x, gridDim.x);
@@ -2811,10 +2907,12 @@ namespace {
 int launch_dispatch_recv(const moe_a2a_shape* s, const void* recv_buf, const int32_t* recv_meta,
                          const int32_t* recv_counts, int32_t rows_hint, int32_t capacity_rows,
                          int32_t* expert_num_tokens, void* expert_x, int32_t* expert_meta,
-                         int32_t* send_back_plan, int32_t* row_position, void* stream) {
+                         int32_t* send_back_plan, int32_t* row_position, void* stream,
+                         int32_t compact_rows = 0, int32_t* expert_offsets = nullptr) {
   if (!shape_ok(s) || rows_hint < 0 || capacity_rows < 0 || !recv_counts || !expert_num_tokens ||
       !expert_x || !expert_meta)
     return MOE_A2A_EINVAL;
+  if (compact_rows > 0 && (!expert_offsets || row_position)) return MOE_A2A_EINVAL;
   if (!counts_fit(capacity_rows, s->world_size)) return MOE_A2A_EINVAL;
   if (rows_hint > capacity_rows) rows_hint = capacity_rows;
   if (capacity_rows > 0 && (!recv_buf || !recv_meta)) return MOE_A2A_EINVAL;
@@ -2836,10 +2934,10 @@ int launch_dispatch_recv(const moe_a2a_shape* s, const void* recv_buf, const int
                                                     capacity_rows, g.nle, g.magic, expert_bits, row_position);
     const int grid = g.nle + mover_blocks(group_items(rows_hint, g));
 #define LAUNCH_P(V, NVW, PLAN)                                                              \
-  dispatch_recv_kernel<V, NVW, PLAN, true><<<grid, 64 * ROWS, 0, st>>>(                     \
+  dispatch_recv_kernel<V, NVW, PLAN, RECV_POS><<<grid, 64 * ROWS, 0, st>>>(                 \
       (const V*)recv_buf, recv_meta, recv_counts, s->world_size, rows_hint, capacity_rows,   \
       g.nle, g.magic, g.max_recv, g.row_vecs, g.wchunks, expert_num_tokens, (V*)expert_x,    \
-      expert_meta, send_back_plan, row_position)
+      expert_meta, send_back_plan, row_position, nullptr)
 #define LAUNCH(V, NVW)                     \
   do {                                     \
     if (planned) LAUNCH_P(V, NVW, true);   \
@@ -2856,15 +2954,20 @@ int launch_dispatch_recv(const moe_a2a_shape* s, const void* recv_buf, const int
   // the stream can hold at most nle * max_recv rows that fit the expert buffers
   if (!items_fit((long long)g.nle * g.max_recv, g.wchunks)) return MOE_A2A_EINVAL;
   const int grid = g.nle + mover_blocks(group_items(rows_hint, g));
-#define LAUNCH_P(V, NVW, PLAN)                                                              \
-  dispatch_recv_kernel<V, NVW, PLAN, false><<<grid, 64 * ROWS, 0, st>>>(                    \
+#define LAUNCH_P(V, NVW, PLAN, MODE)                                                        \
+  dispatch_recv_kernel<V, NVW, PLAN, MODE><<<grid, 64 * ROWS, 0, st>>>(                     \
       (const V*)recv_buf, recv_meta, recv_counts, s->world_size, rows_hint, capacity_rows,   \
-      g.nle, g.magic, g.max_recv, g.row_vecs, g.wchunks, expert_num_tokens, (V*)expert_x,    \
-      expert_meta, send_back_plan, nullptr)
-#define LAUNCH(V, NVW)                     \
-  do {                                     \
-    if (planned) LAUNCH_P(V, NVW, true);   \
-    else LAUNCH_P(V, NVW, false);          \
+      g.nle, g.magic, compact_rows > 0 ? compact_rows : g.max_recv, g.row_vecs, g.wchunks,   \
+      expert_num_tokens, (V*)expert_x, expert_meta, send_back_plan, nullptr, expert_offsets)
+#define LAUNCH(V, NVW)                                         \
+  do {                                                         \
+    if (compact_rows > 0) {                                    \
+      if (planned) LAUNCH_P(V, NVW, true, RECV_COMPACT);       \
+      else LAUNCH_P(V, NVW, false, RECV_COMPACT);              \
+    } else {                                                   \
+      if (planned) LAUNCH_P(V, NVW, true, RECV_SCAN);          \
+      else LAUNCH_P(V, NVW, false, RECV_SCAN);                 \
+    }                                                          \
   } while (0)
   MOE_A2A_FOR_WAVE_KERNEL(g, LAUNCH);
 #undef LAUNCH
@@ -2911,17 +3014,26 @@ int moe_a2a_dispatch_recv_static(const moe_a2a_shape* s, const void* recv_buf,
   return rc;
 }
 
-int moe_a2a_combine_send(const moe_a2a_shape* s, const void* expert_y, const int32_t* expert_meta,
-                         const int32_t* expert_num_tokens, int32_t rows_hint,
-                         int32_t capacity_rows, void* send_buf, int32_t* send_meta, int32_t* send_counts,
-                         const int32_t* send_back_plan, void* stream) {
-  if (!shape_ok(s) || rows_hint < 0 || capacity_rows < 0 || !expert_y || !expert_meta ||
+}  // extern "C"
+
+namespace {
+
+// Stage 3; compact_rows > 0: the expert buffers hold the experts' rows back to back.
+int launch_combine_send(const moe_a2a_shape* s, const void* expert_y, const int32_t* expert_meta,
+                        const int32_t* expert_num_tokens, int32_t rows_hint, int32_t capacity_rows,
+                        void* send_buf, int32_t* send_meta, int32_t* send_counts,
+                        const int32_t* send_back_plan, int32_t compact_rows, void* stream) {
+  if (!shape_ok(s) || rows_hint < 0 || capacity_rows < 0 || compact_rows < 0 || !expert_y || !expert_meta ||
       !expert_num_tokens || !send_counts)
     return MOE_A2A_EINVAL;
   if (capacity_rows > 0 && (!send_buf || !send_meta)) return MOE_A2A_EINVAL;
   if (!all_aligned(2, expert_y, send_buf)) return MOE_A2A_EALIGN;
   Geometry g = geometry(s, expert_y, send_buf);
   if (g.nle > MAX_LOCAL_EXPERTS) return MOE_A2A_EINVAL;
+  if (compact_rows > 0) {
+    if (!counts_fit(compact_rows, g.nle)) return MOE_A2A_EINVAL;  // counts cut to the capacity add up in an int
+    g.max_recv = compact_rows;  // no expert has more rows than the buffers hold
+  }
   const bool planned = send_back_plan && plan_supported(s);
   // The planned path has no scan to repeat per chunk, so a row can be split among more waves:
   // 4 vectors per lane (a 256-vector chunk per wave) made the whole step 0.5 us shorter at
@@ -2930,14 +3042,15 @@ int moe_a2a_combine_send(const moe_a2a_shape* s, const void* expert_y, const int
     g.nvw = MOE_A2A_PLANNED_NVW;
     g.wchunks = (g.row_vecs + 64 * g.nvw - 1) / (64 * g.nvw);
   }
-  if (!items_fit((long long)g.nle * g.max_recv, g.wchunks)) return MOE_A2A_EINVAL;
+  if (!items_fit(compact_rows > 0 ? (long long)compact_rows : (long long)g.nle * g.max_recv, g.wchunks))
+    return MOE_A2A_EINVAL;
   const int grid = s->world_size + mover_blocks(group_items(rows_hint, g));
   hipStream_t st = (hipStream_t)stream;
 #define LAUNCH_S(V, NVW, SMALL, PLAN)                                                          \
   combine_send_kernel<V, NVW, SMALL, PLAN><<<grid, 64 * ROWS, 0, st>>>(                       \
       (const V*)expert_y, expert_meta, expert_num_tokens, g.nle, g.max_recv, s->world_size,    \
       g.row_vecs, g.wchunks, capacity_rows, (V*)send_buf, send_meta, send_counts,              \
-      send_back_plan)
+      send_back_plan, compact_rows)
 #define LAUNCH(V, NVW)                                   \
   do {                                                   \
     if (planned) LAUNCH_S(V, NVW, true, true);           \
@@ -2949,10 +3062,6 @@ int moe_a2a_combine_send(const moe_a2a_shape* s, const void* expert_y, const int
 #undef LAUNCH_S
   return launch_status();
 }
-
-}  // extern "C"
-
-namespace {
 
 // Stage 4; with `entry_row` (num_tokens * K ints of workspace) a launch of its own first maps
 // every (token, k) to its arriving row and the workgroups look their rows up instead of scanning.
@@ -3022,6 +3131,35 @@ int launch_combine_recv(const moe_a2a_shape* s, const void* recv_buf, const int3
 
 extern "C" {
 
+int moe_a2a_dispatch_recv_compact(const moe_a2a_shape* s, const void* recv_buf, const int32_t* recv_meta,
+                                  const int32_t* recv_counts, int32_t rows_hint, int32_t capacity_rows,
+                                  int32_t* expert_num_tokens, int32_t* expert_offsets, void* expert_x,
+                                  int32_t* expert_meta, int32_t compact_capacity_rows,
+                                  int32_t* send_back_plan, void* stream) {
+  if (compact_capacity_rows < 1 || !expert_offsets) return MOE_A2A_EINVAL;
+  return launch_dispatch_recv(s, recv_buf, recv_meta, recv_counts, rows_hint, capacity_rows, expert_num_tokens,
+                              expert_x, expert_meta, send_back_plan, nullptr, stream, compact_capacity_rows,
+                              expert_offsets);
+}
+
+int moe_a2a_combine_send(const moe_a2a_shape* s, const void* expert_y, const int32_t* expert_meta,
+                         const int32_t* expert_num_tokens, int32_t rows_hint,
+                         int32_t capacity_rows, void* send_buf, int32_t* send_meta, int32_t* send_counts,
+                         const int32_t* send_back_plan, void* stream) {
+  return launch_combine_send(s, expert_y, expert_meta, expert_num_tokens, rows_hint, capacity_rows, send_buf,
+                             send_meta, send_counts, send_back_plan, 0, stream);
+}
+
+int moe_a2a_combine_send_compact(const moe_a2a_shape* s, const void* expert_y, const int32_t* expert_meta,
+                                 const int32_t* expert_num_tokens, int32_t rows_hint,
+                                 int32_t compact_capacity_rows, int32_t capacity_rows, void* send_buf,
+                                 int32_t* send_meta, int32_t* send_counts, const int32_t* send_back_plan,
+                                 void* stream) {
+  if (compact_capacity_rows < 1) return MOE_A2A_EINVAL;
+  return launch_combine_send(s, expert_y, expert_meta, expert_num_tokens, rows_hint, capacity_rows, send_buf,
+                             send_meta, send_counts, send_back_plan, compact_capacity_rows, stream);
+}
+
 int moe_a2a_combine_recv(const moe_a2a_shape* s, const void* recv_buf, const int32_t* recv_meta,
                          const int32_t* recv_counts, int32_t rows_hint, int32_t capacity_rows,
                          const float* weights, int32_t num_tokens, void* out_tokens,
@@ -3039,18 +3177,28 @@ int moe_a2a_combine_recv_long(const moe_a2a_shape* s, const void* recv_buf, cons
                              num_tokens, out_tokens, accumulate, dtype, entry_row, stream);
 }
 
-int moe_a2a_expert_scale(const moe_a2a_shape* s, const void* expert_x,
-                         const int32_t* expert_num_tokens, int32_t rows_hint, int32_t in_dtype,
-                         int32_t out_dtype, void* expert_y, void* stream) {
-  if (!shape_ok(s) || rows_hint < 0 || !expert_x || !expert_num_tokens || !expert_y)
+}  // extern "C"
+
+namespace {
+
+// The stand-in expert; compact_rows > 0: the expert buffers hold the experts' rows back to back.
+int launch_expert_scale(const moe_a2a_shape* s, const void* expert_x, const int32_t* expert_num_tokens,
+                        int32_t rows_hint, int32_t in_dtype, int32_t out_dtype, void* expert_y,
+                        int32_t compact_rows, void* stream) {
+  if (!shape_ok(s) || rows_hint < 0 || compact_rows < 0 || !expert_x || !expert_num_tokens || !expert_y)
     return MOE_A2A_EINVAL;
   if ((in_dtype != MOE_A2A_F16 && in_dtype != MOE_A2A_BF16) ||
       (out_dtype != MOE_A2A_F16 && out_dtype != MOE_A2A_BF16))
     return MOE_A2A_EINVAL;
   if (!all_aligned(2, expert_x, expert_y)) return MOE_A2A_EALIGN;
-  const Geometry g = geometry(s, expert_x, expert_y);
+  Geometry g = geometry(s, expert_x, expert_y);
   if (g.nle > MAX_LOCAL_EXPERTS) return MOE_A2A_EINVAL;
-  if (!items_fit((long long)g.nle * g.max_recv, g.chunks)) return MOE_A2A_EINVAL;
+  if (compact_rows > 0) {
+    if (!counts_fit(compact_rows, g.nle)) return MOE_A2A_EINVAL;
+    g.max_recv = compact_rows;
+  }
+  const long long most_rows = compact_rows > 0 ? (long long)compact_rows : (long long)g.nle * g.max_recv;
+  if (!items_fit(most_rows, g.chunks)) return MOE_A2A_EINVAL;
   hipStream_t st = (hipStream_t)stream;
   const float scale = (float)(1 + s->rank);
 #ifndef MOE_A2A_SCALE_WAVES
@@ -3059,12 +3207,12 @@ int moe_a2a_expert_scale(const moe_a2a_shape* s, const void* expert_x,
   if (MOE_A2A_SCALE_WAVES && g.vec16 && g.nle <= 64) {
     const int nvw = g.nvw < 4 ? g.nvw : 4;  // 1, 2 or 4 vectors per lane
     const int wchunks = (g.row_vecs + 64 * nvw - 1) / (64 * nvw);
-    if (!items_fit((long long)g.nle * g.max_recv, wchunks)) return MOE_A2A_EINVAL;
+    if (!items_fit(most_rows, wchunks)) return MOE_A2A_EINVAL;
     const int wgrid = mover_blocks(((long long)rows_hint * wchunks + ROWS - 1) / ROWS);
 #define LAUNCH_WT(NVW, DI, DO)                                                                 \
   expert_scale_wave_kernel<NVW, DI, DO><<<wgrid, 64 * ROWS, 0, st>>>(                          \
       (const b128*)expert_x, expert_num_tokens, g.nle, g.max_recv, scale, g.row_vecs, wchunks,  \
-      (b128*)expert_y)
+      (b128*)expert_y, compact_rows)
 #define LAUNCH_W(NVW)                                                                          \
   do {                                                                                         \
     if (in_dtype == MOE_A2A_BF16 && out_dtype == MOE_A2A_BF16)                                 \
@@ -3087,7 +3235,7 @@ int moe_a2a_expert_scale(const moe_a2a_shape* s, const void* expert_x,
 #define LAUNCH_T(V, NV, DI, DO)                                                              \
   expert_scale_kernel<V, NV, DI, DO><<<grid, BLOCK, 0, st>>>(                                \
       (const V*)expert_x, expert_num_tokens, g.nle, g.max_recv, scale, g.row_vecs, g.chunks, \
-      (V*)expert_y)
+      (V*)expert_y, compact_rows)
 #define LAUNCH(V, NV)                                                                         \
   do {                                                                                        \
     if (in_dtype == MOE_A2A_BF16 && out_dtype == MOE_A2A_BF16)                                \
@@ -3105,6 +3253,25 @@ int moe_a2a_expert_scale(const moe_a2a_shape* s, const void* expert_x,
   return launch_status();
 }
 
+}  // namespace
+
+extern "C" {
+
+int moe_a2a_expert_scale(const moe_a2a_shape* s, const void* expert_x,
+                         const int32_t* expert_num_tokens, int32_t rows_hint, int32_t in_dtype,
+                         int32_t out_dtype, void* expert_y, void* stream) {
+  return launch_expert_scale(s, expert_x, expert_num_tokens, rows_hint, in_dtype, out_dtype, expert_y, 0, stream);
+}
+
+int moe_a2a_expert_scale_compact(const moe_a2a_shape* s, const void* expert_x,
+                                 const int32_t* expert_num_tokens, int32_t rows_hint,
+                                 int32_t compact_capacity_rows, int32_t in_dtype, int32_t out_dtype,
+                                 void* expert_y, void* stream) {
+  if (compact_capacity_rows < 1) return MOE_A2A_EINVAL;
+  return launch_expert_scale(s, expert_x, expert_num_tokens, rows_hint, in_dtype, out_dtype, expert_y,
+                             compact_capacity_rows, stream);
+}
+
 #ifndef MOE_A2A_GEMM_ROWS_FOR_128
 #define MOE_A2A_GEMM_ROWS_FOR_128 48  // rows per group (mean, from the hint) above which blocks hold 128 tokens
 #endif
@@ -3117,7 +3284,7 @@ namespace {
 // rows; rows_of_group null means max_rows rows in every group.
 int launch_grouped_gemm(const void* x, const int32_t* rows_of_group, const void* w, const void* bias,
                         void* y, int groups, long long max_rows, long long rows_hint, int N, int K,
-                        int dtype, hipStream_t st) {
+                        int dtype, hipStream_t st, int compact = 0) {
   if (dtype != MOE_A2A_F16 && dtype != MOE_A2A_BF16) return MOE_A2A_EINVAL;
   if (N % 32 != 0 || K % 8 != 0) return MOE_A2A_EINVAL;  // whole wave tiles of columns, whole 16-byte vectors
   if (!all_aligned(16, x, w, y) || !all_aligned(8, bias)) return MOE_A2A_EALIGN;
@@ -3154,7 +3321,7 @@ int launch_grouped_gemm(const void* x, const int32_t* rows_of_group, const void*
 #define LAUNCH_G(DT, TJ, GW)                                                                          \
   expert_gemm_kernel<DT, TJ, GW><<<grid, 64 * GW, 0, st>>>((const b128*)x, rows_of_group, (const b128*)w, \
                                                            (const uint16_t*)bias, (uint16_t*)y, groups,  \
-                                                           (int)max_rows, N, K, col_tiles)
+                                                           (int)max_rows, N, K, col_tiles, compact)
 #define LAUNCH_GW(DT)                                 \
   do {                                                \
     if (tj == 2) LAUNCH_G(DT, 2, 4);                  \
@@ -3250,7 +3417,7 @@ int launch_dense_gemm(const void* a, const void* b, const void* bias, void* c, i
 #define LAUNCH_D(DT, TM, TN)                                                             \
   dense_gemm_kernel<DT, 2, 2, TM, TN, false><<<grid, 256, lds_bytes, st>>>(              \
       (const b128*)a, (const b128*)b, (const uint16_t*)bias, (uint16_t*)c, M, N, K, (int)tiles_m, (int)tiles_n, \
-      nullptr, 0, 0)
+      nullptr, 0, 0, 0)
 #define LAUNCH_DT(DT)                         \
   do {                                        \
     if (tile == 256) LAUNCH_D(DT, 4, 4);      \
@@ -3277,7 +3444,7 @@ int launch_dense_gemm(const void* a, const void* b, const void* bias, void* c, i
 // LDS) do better than the kernel that is built around streaming. MOE_A2A_NOT_DENSE otherwise.
 int launch_grouped_dense(const void* x, const int32_t* rows_of_group, const void* w, const void* bias, void* y,
                          int groups, long long max_rows, long long rows_hint, int N, int K, int dtype,
-                         hipStream_t st) {
+                         hipStream_t st, int compact = 0) {
   if (dtype != MOE_A2A_F16 && dtype != MOE_A2A_BF16) return MOE_A2A_EINVAL;
   if (N % 32 != 0 || K % 8 != 0) return MOE_A2A_EINVAL;
   if (!all_aligned(16, x, w, y) || !all_aligned(8, bias)) return MOE_A2A_EALIGN;
@@ -3302,7 +3469,7 @@ int launch_grouped_dense(const void* x, const int32_t* rows_of_group, const void
 #define LAUNCH_GD(DT, TM, TN)                                                                 \
   dense_gemm_kernel<DT, 2, 2, TM, TN, true><<<grid, 256, lds_bytes, st>>>(                    \
       (const b128*)x, (const b128*)w, (const uint16_t*)bias, (uint16_t*)y, 0, N, K, 0, (int)tiles_n,        \
-      rows_of_group, groups, (int)max_rows)
+      rows_of_group, groups, (int)max_rows, compact)
   if (dtype == MOE_A2A_BF16) {
     if (tile == 256) LAUNCH_GD(MOE_A2A_BF16, 4, 4);
     else if (tile == 128) LAUNCH_GD(MOE_A2A_BF16, 2, 2);
@@ -3376,6 +3543,25 @@ int moe_a2a_expert_gemm(const moe_a2a_shape* s, const void* expert_x,
   if (dense != MOE_A2A_NOT_DENSE) return dense;
   return launch_grouped_gemm(expert_x, expert_num_tokens, weights, bias, expert_y, nle, max_recv, rows_hint,
                              out_dim, in_dim, dtype, (hipStream_t)stream);
+}
+
+int moe_a2a_expert_gemm_compact(const moe_a2a_shape* s, const void* expert_x,
+                                const int32_t* expert_num_tokens, int32_t rows_hint,
+                                int32_t compact_capacity_rows, const void* weights, const void* bias,
+                                int32_t in_dim, int32_t out_dim, int32_t dtype, void* expert_y,
+                                void* stream) {
+  if (!shape_ok(s) || rows_hint < 0 || compact_capacity_rows < 1 || in_dim < 1 || out_dim < 1 || !expert_x ||
+      !expert_num_tokens || !weights || !expert_y)
+    return MOE_A2A_EINVAL;
+  const int nle = s->num_experts / s->world_size;
+  if (!counts_fit(compact_capacity_rows, nle)) return MOE_A2A_EINVAL;
+  // (every count is cut to the rows the buffers hold; counts that dispatch_recv_compact wrote add up to at most that)
+  const int dense = launch_grouped_dense(expert_x, expert_num_tokens, weights, bias, expert_y, nle,
+                                         compact_capacity_rows, rows_hint, out_dim, in_dim, dtype,
+                                         (hipStream_t)stream, 1);
+  if (dense != MOE_A2A_NOT_DENSE) return dense;
+  return launch_grouped_gemm(expert_x, expert_num_tokens, weights, bias, expert_y, nle, compact_capacity_rows,
+                             rows_hint, out_dim, in_dim, dtype, (hipStream_t)stream, 1);
 }
 
 int moe_a2a_linear(const void* input, const void* weight, const void* bias, int32_t m, int32_t n,

@@ -305,3 +305,106 @@ void a2a_exchange_gather_local(int64_t world_size, int64_t hidden_dim, std::vect
                                        to_i32(recv_capacity, "recv_capacity_rows"), stream_of(stream)),
          "moe_a2a_exchange_gather_local");
 }
+
+// ---- the compact expert-major layout: 2-D expert buffers [rows, width], the experts' rows back to back
+
+namespace {
+int64_t compact_rows(const torch::Tensor& rows, const char* what) {
+  TORCH_CHECK(rows.dim() == 2 && rows.size(0) >= 1, what, ": compact expert buffers are [rows, width] with rows >= 1");
+  return rows.size(0);
+}
+}  // namespace
+
+void a2a_dispatch_recv_compact(std::vector<int64_t> shape, torch::Tensor recv_buf, torch::Tensor recv_meta,
+                               torch::Tensor recv_counts, int64_t rows_hint, torch::Tensor expert_num_tokens,
+                               torch::Tensor expert_offsets, torch::Tensor expert_x, torch::Tensor expert_meta,
+                               c10::optional<torch::Tensor> send_back_plan, int64_t stream) {
+  const moe_a2a_shape s = shape_of(shape);
+  const auto dt = rows_type(recv_buf, "recv_buf");
+  const int64_t nle = s.world_size > 0 ? s.num_experts / s.world_size : 0;
+  need(recv_buf, "recv_buf", dt, 0);
+  need(recv_meta, "recv_meta", torch::kInt32, 0, &recv_buf);
+  const int64_t capacity = std::min(recv_buf.numel() / std::max<int64_t>(s.hidden_dim, 1),
+                                    recv_meta.numel() / MOE_A2A_META_DIM);
+  const int64_t room = std::min(compact_rows(expert_x, "expert_x"), compact_rows(expert_meta, "expert_meta"));
+  need(recv_counts, "recv_counts", torch::kInt32, s.world_size, &recv_buf);
+  need(expert_num_tokens, "expert_num_tokens", torch::kInt32, nle, &recv_buf);
+  need(expert_offsets, "expert_offsets", torch::kInt32, nle + 1, &recv_buf);
+  need(expert_x, "expert_x", dt, room * s.hidden_dim, &recv_buf);
+  need(expert_meta, "expert_meta", torch::kInt32, room * MOE_A2A_META_DIM, &recv_buf);
+  if (send_back_plan.has_value())
+    need(*send_back_plan, "send_back_plan", torch::kInt32, 2 * (int64_t)s.num_experts, &recv_buf);
+  status(moe_a2a_dispatch_recv_compact(&s, recv_buf.data_ptr(), ints(recv_meta), ints(recv_counts),
+                                       to_i32(std::min(rows_hint, capacity), "rows_hint"),
+                                       to_i32(capacity, "capacity_rows"), ints(expert_num_tokens),
+                                       ints(expert_offsets), expert_x.data_ptr(), ints(expert_meta),
+                                       to_i32(room, "compact_capacity_rows"), ints_or_null(send_back_plan),
+                                       stream_of(stream)),
+         "moe_a2a_dispatch_recv_compact");
+}
+
+void a2a_expert_scale_compact(std::vector<int64_t> shape, torch::Tensor expert_x, torch::Tensor expert_num_tokens,
+                              int64_t rows_hint, torch::Tensor expert_y, int64_t stream) {
+  const moe_a2a_shape s = shape_of(shape);
+  const auto din = rows_type(expert_x, "expert_x"), dout = rows_type(expert_y, "expert_y");
+  const int64_t nle = s.world_size > 0 ? s.num_experts / s.world_size : 0;
+  const int64_t room = std::min(compact_rows(expert_x, "expert_x"), compact_rows(expert_y, "expert_y"));
+  need(expert_x, "expert_x", din, room * s.hidden_dim);
+  need(expert_y, "expert_y", dout, room * s.hidden_dim, &expert_x);
+  need(expert_num_tokens, "expert_num_tokens", torch::kInt32, nle, &expert_x);
+  status(moe_a2a_expert_scale_compact(&s, expert_x.data_ptr(), ints(expert_num_tokens),
+                                      to_i32(rows_hint, "rows_hint"), to_i32(room, "compact_capacity_rows"),
+                                      dtype_code(din), dtype_code(dout), expert_y.data_ptr(), stream_of(stream)),
+         "moe_a2a_expert_scale_compact");
+}
+
+void a2a_expert_gemm_compact(std::vector<int64_t> shape, torch::Tensor expert_x, torch::Tensor expert_num_tokens,
+                             int64_t rows_hint, torch::Tensor weights, c10::optional<torch::Tensor> bias,
+                             torch::Tensor expert_y, int64_t stream) {
+  const moe_a2a_shape s = shape_of(shape);
+  const auto dt = rows_type(expert_x, "expert_x");
+  const int64_t nle = s.world_size > 0 ? s.num_experts / s.world_size : 0;
+  TORCH_CHECK(weights.dim() == 3 && weights.size(0) == nle, "weights must be [num_local_experts, out_dim, in_dim]");
+  const int64_t out_dim = weights.size(1), in_dim = weights.size(2);
+  const int64_t room = std::min(compact_rows(expert_x, "expert_x"), compact_rows(expert_y, "expert_y"));
+  need(expert_x, "expert_x", dt, room * in_dim);
+  need(expert_y, "expert_y", dt, room * out_dim, &expert_x);
+  need(weights, "weights", dt, nle * out_dim * in_dim, &expert_x);
+  need(expert_num_tokens, "expert_num_tokens", torch::kInt32, nle, &expert_x);
+  const void* b = nullptr;
+  if (bias.has_value()) {
+    need(*bias, "bias", dt, nle * out_dim, &expert_x);
+    b = bias->data_ptr();
+  }
+  status(moe_a2a_expert_gemm_compact(&s, expert_x.data_ptr(), ints(expert_num_tokens), to_i32(rows_hint, "rows_hint"),
+                                     to_i32(room, "compact_capacity_rows"), weights.data_ptr(), b,
+                                     to_i32(in_dim, "in_dim"), to_i32(out_dim, "out_dim"), dtype_code(dt),
+                                     expert_y.data_ptr(), stream_of(stream)),
+         "moe_a2a_expert_gemm_compact");
+}
+
+void a2a_combine_send_compact(std::vector<int64_t> shape, torch::Tensor expert_y, torch::Tensor expert_meta,
+                              torch::Tensor expert_num_tokens, int64_t rows_hint, torch::Tensor send_buf,
+                              torch::Tensor send_meta, torch::Tensor send_counts,
+                              c10::optional<torch::Tensor> send_back_plan, int64_t stream) {
+  const moe_a2a_shape s = shape_of(shape);
+  const auto dt = rows_type(expert_y, "expert_y");
+  const int64_t nle = s.world_size > 0 ? s.num_experts / s.world_size : 0;
+  const int64_t room = std::min(compact_rows(expert_y, "expert_y"), compact_rows(expert_meta, "expert_meta"));
+  need(expert_y, "expert_y", dt, room * s.hidden_dim);
+  need(expert_meta, "expert_meta", torch::kInt32, room * MOE_A2A_META_DIM, &expert_y);
+  need(expert_num_tokens, "expert_num_tokens", torch::kInt32, nle, &expert_y);
+  need(send_buf, "send_buf", dt, 0, &expert_y);
+  need(send_meta, "send_meta", torch::kInt32, 0, &expert_y);
+  const int64_t capacity = std::min(send_buf.numel() / std::max<int64_t>(s.hidden_dim, 1),
+                                    send_meta.numel() / MOE_A2A_META_DIM);
+  need(send_counts, "send_counts", torch::kInt32, s.world_size, &expert_y);
+  if (send_back_plan.has_value())
+    need(*send_back_plan, "send_back_plan", torch::kInt32, 2 * (int64_t)s.num_experts, &expert_y);
+  status(moe_a2a_combine_send_compact(&s, expert_y.data_ptr(), ints(expert_meta), ints(expert_num_tokens),
+                                      to_i32(std::min(rows_hint, capacity), "rows_hint"),
+                                      to_i32(room, "compact_capacity_rows"), to_i32(capacity, "capacity_rows"),
+                                      send_buf.data_ptr(), ints(send_meta), ints(send_counts),
+                                      ints_or_null(send_back_plan), stream_of(stream)),
+         "moe_a2a_combine_send_compact");
+}

@@ -402,6 +402,78 @@ int moe_a2a_exchange_local(int32_t world_size, int32_t hidden_dim,
                            int32_t recv_capacity_rows, void* stream);
 
 /*
+ * The compact expert-major layout: the four entry points between the two
+ * exchanges with the experts' rows back to back instead of in the reference's
+ * padded buffers. all2all/reference.py:123-136 allocates
+ * expert_x[nle, max_recv, H] and expert_meta[nle, max_recv, 5] with
+ * max_recv = max_num_tokens * world_size rows for EVERY local expert (939 MB per
+ * buffer at 32 experts, 2048 rows, hidden_dim 7168) and fills what arrives
+ * (about 29 MB of it). Here row pos of local expert le lies at row
+ *   expert_offsets[le] + pos
+ * of buffers of compact_capacity_rows rows, with expert_offsets the exclusive
+ * prefix of the rows per expert; the order of the rows (le ascending, arrival
+ * order inside an expert) is the reference's. Expanding the compact buffers to
+ * the padded ones reproduces what moe_a2a_dispatch_recv writes, row for row.
+ *
+ * compact_capacity_rows is the caller's choice: at least the rows the rank
+ * receives (max_num_tokens * world_size * min(experts_per_token, nle) always
+ * suffices; balanced routing delivers about max_num_tokens * experts_per_token).
+ * Rows that find no room are not stored (they are the last of the (le, pos)
+ * order); expert_num_tokens still reports every row that arrived, as in the
+ * padded layout, and the three consumers below cut the counts they are given
+ * to the rows that fit, so counts that add up to more than the buffers hold
+ * never send a load or a store past their end. send_back_plan is used as in
+ * the padded entry points (moe_a2a_combine_send_compact sets it aside by itself
+ * when rows found no room).
+ *
+ * moe_a2a_dispatch_recv_compact: as moe_a2a_dispatch_recv, plus
+ *   expert_offsets  int32[nle + 1] out: first row of every expert, the exclusive
+ *                   prefix of expert_num_tokens; [nle] = rows that arrived
+ *   expert_x        [compact_capacity_rows, H], expert_meta [compact_capacity_rows, 5]
+ * Every mover workgroup counts the rows of lower experts over the whole stream
+ * (one pass over all keys instead of the keys ahead of it), so this entry point
+ * is meant for the streams of a few thousand rows the one-launch entry points
+ * serve; there is no long-stream form of it.
+ */
+int moe_a2a_dispatch_recv_compact(const moe_a2a_shape* shape, const void* recv_buf,
+                                  const int32_t* recv_meta, const int32_t* recv_counts,
+                                  int32_t rows_hint, int32_t capacity_rows,
+                                  int32_t* expert_num_tokens, int32_t* expert_offsets,
+                                  void* expert_x, int32_t* expert_meta,
+                                  int32_t compact_capacity_rows, int32_t* send_back_plan,
+                                  void* stream);
+
+/* moe_a2a_expert_scale on compact buffers: expert_x, expert_y [compact_capacity_rows, H]. */
+int moe_a2a_expert_scale_compact(const moe_a2a_shape* shape, const void* expert_x,
+                                 const int32_t* expert_num_tokens, int32_t rows_hint,
+                                 int32_t compact_capacity_rows, int32_t in_dtype,
+                                 int32_t out_dtype, void* expert_y, void* stream);
+
+/*
+ * moe_a2a_expert_gemm on compact buffers: expert_x [compact_capacity_rows, in_dim],
+ * expert_y [compact_capacity_rows, out_dim]; row j of expert le is row
+ * (rows of the experts below le) + j of both. The same kernels, limits and
+ * arithmetic; which layout the rows lie in changes no bit of a result.
+ */
+int moe_a2a_expert_gemm_compact(const moe_a2a_shape* shape, const void* expert_x,
+                                const int32_t* expert_num_tokens, int32_t rows_hint,
+                                int32_t compact_capacity_rows, const void* weights,
+                                const void* bias, int32_t in_dim, int32_t out_dim,
+                                int32_t dtype, void* expert_y, void* stream);
+
+/*
+ * moe_a2a_combine_send on compact buffers: expert_y [compact_capacity_rows, H],
+ * expert_meta [compact_capacity_rows, 5] as moe_a2a_dispatch_recv_compact left
+ * them; capacity_rows is that of send_buf / send_meta as before.
+ */
+int moe_a2a_combine_send_compact(const moe_a2a_shape* shape, const void* expert_y,
+                                 const int32_t* expert_meta, const int32_t* expert_num_tokens,
+                                 int32_t rows_hint, int32_t compact_capacity_rows,
+                                 int32_t capacity_rows, void* send_buf, int32_t* send_meta,
+                                 int32_t* send_counts, const int32_t* send_back_plan,
+                                 void* stream);
+
+/*
  * The same stand-in for every source of one destination rank in one launch:
  * what the three dist.all_to_all_single calls at all2all/reference.py:88-91 and
  * :107-119 (dispatch), :181-185 and :210-222 (combine) deliver to ONE rank.
