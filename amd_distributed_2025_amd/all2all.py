@@ -289,10 +289,18 @@ class HIPAllToAll:
              plan, _stream(self.device))
         return counts, buf, meta
 
-    def combine_recv(self, out_tokens, weights, ret_counts, ret_buf, ret_meta, accumulate: bool = True):
+    def combine_recv(self, out_tokens, weights, ret_counts, ret_buf, ret_meta, accumulate: bool = True,
+                     unique_pairs: bool = True):
         """`out_tokens[t] += row.float() * weights[t, k]` for the arriving rows, in
         arrival order, rounding to out_dtype after every addend. With
-        `accumulate=False` the sum starts from zero and `out_tokens` is only written."""
+        `accumulate=False` the sum starts from zero and `out_tokens` is only written.
+
+        Streams of more than `LONG_STREAM_ROWS["combine"]` rows go through a (token, k) -> row
+        table, which holds ONE row per pair: every stream a dispatch produced has each pair once,
+        and for those the result is the same. A caller that feeds a stream in which a (src_token,
+        src_k) pair may arrive more than once (the reference, all2all/reference.py:227-232, adds
+        every arriving row) says so with `unique_pairs=False`; the rows are then found by scanning
+        whatever the length, and every one of them is added."""
         cfg = self.cfg
         _need(out_tokens, cfg.out_dtype, self.device, "out_tokens")
         _need(weights, torch.float32, self.device, "weights")
@@ -305,7 +313,7 @@ class HIPAllToAll:
         capacity = min(ret_buf.shape[0], ret_meta.shape[0])
         hint = min(capacity, T * cfg.experts_per_token)
         table = None
-        if hint > self._long_from("combine"):
+        if unique_pairs and hint > self._long_from("combine"):
             table = self._buf("entry_row", (cfg.max_num_tokens * cfg.experts_per_token,), torch.int32)
         self.binding.combine_recv(self.shape, ret_buf, ret_meta, ret_counts, hint, weights, T, out_tokens,
                                   accumulate, _stream(self.device), table)

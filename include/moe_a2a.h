@@ -364,7 +364,8 @@ int moe_a2a_expert_gemm(const moe_a2a_shape* shape, const void* expert_x,
  * rounded value and the sum rounded again, which is what the two torch
  * statements do. bias may be NULL.
  * One of three kernels runs, picked from the shape alone (so a shape always
- * gives the same bits): up to 64 rows and from 512 elements of k, a kernel whose
+ * gives the same bits): for m <= 64, k >= 449 (eight steps of 64 elements) and
+ * n <= 24448 (fewer than 192 tiles of 128 columns), a kernel whose
  * workgroups own 32 columns and split k over their waves (partial sums added in
  * a fixed order); else a kernel bound by the matrix cores, whose workgroups own
  * output tiles of 256 x 256, 128 x 128 or 64 x 128 (the largest that still

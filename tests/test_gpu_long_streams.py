@@ -235,3 +235,42 @@ def test_counts_beyond_capacity_are_cut_off_by_the_long_stream_entry_points():
                                           None, None, st) == -1
     assert lib.moe_a2a_combine_recv_long(shape, p(recv_buf), p(recv_meta), p(counts40), CAP, CAP, p(weights), max_T,
                                          p(y), 0, _lib.BF16, None, st) == -1
+
+
+def test_a_pair_that_arrives_twice_is_added_twice_only_when_the_caller_says_pairs_may_repeat():
+    """The reference adds every arriving row (all2all/reference.py:227-232). A stream out of a
+    dispatch has every (src_token, src_k) pair once; a caller-made stream in which one repeats is
+    served by the scan (`unique_pairs=False`), which adds both rows whatever the length. The table of
+    the long-stream entry point holds one row per pair: by default, above its threshold, exactly one
+    of the two rows is added."""
+    from amd_distributed_2025_amd import HIPAllToAll
+    from amd_distributed_2025_amd.task import MoEConfig
+    from oracle import moe_a2a_oracle as orc
+
+    T, K, H, W = 640, 8, 64, 1
+    cfg = MoEConfig(8, K, H, T, torch.bfloat16, torch.bfloat16)
+    a = HIPAllToAll(cfg, 0, W, device=DEV)
+    rng = np.random.default_rng(5)
+    S = T * K
+    assert S > LONG_STREAM_ROWS["combine"]
+    order = rng.permutation(S)
+    meta = np.zeros((S + 1, 5), np.int32)
+    meta[:S, 2], meta[:S, 3] = order // K, order % K
+    dup = 1234
+    meta[S] = meta[dup]                              # the pair of row `dup` arrives again at the end
+    rows = torch.from_numpy(rng.standard_normal((S + 1, H)).astype(np.float32)).to(torch.bfloat16)
+    weights = torch.from_numpy(rng.random((T, K), dtype=np.float32))
+    counts = torch.tensor([S + 1], dtype=torch.int32, device=DEV)
+    y = torch.empty(T, H, dtype=torch.bfloat16, device=DEV)
+    args = (weights.to(DEV), counts, rows.to(DEV), torch.from_numpy(meta).to(DEV))
+    both = orc.combine_recv(bits(rows), meta, weights.numpy(), T, "bf16")
+    a.combine_recv(y, *args, accumulate=False, unique_pairs=False)
+    torch.cuda.synchronize()
+    assert np.array_equal(bits(y), both)
+    a.combine_recv(y, *args, accumulate=False)       # by default: the table, one row per pair
+    torch.cuda.synchronize()
+    keep_first, keep_last = np.ones(S + 1, bool), np.ones(S + 1, bool)
+    keep_first[S], keep_last[dup] = False, False
+    one_of = [orc.combine_recv(bits(rows)[k], meta[k], weights.numpy(), T, "bf16") for k in (keep_first, keep_last)]
+    assert any(np.array_equal(bits(y), w) for w in one_of)
+    assert not np.array_equal(bits(y), both)

@@ -22,14 +22,17 @@ SMALL = dict(world_size=4, num_experts=8, experts_per_token=2, hidden_dim=264, m
              num_tokens="full", routing="uniform", weights="rand", dtype="fp16")
 
 
+class _RawInts:
+    """n int32 at a raw device address, for torch.as_tensor (the array interface torch reads)."""
+
+    def __init__(self, address: int, n: int):
+        self.__cuda_array_interface__ = {"shape": (n,), "typestr": "<i4", "data": (address, False), "version": 2}
+
+
 def device_ints(address: int, n: int) -> np.ndarray:
-    """Copy n int32 from a raw device address to the host (the plan lives in memory torch does not own)."""
-    out = torch.empty(n, dtype=torch.int32, device=DEV)
-    hip = C.CDLL("libamdhip64.so")
-    hip.hipMemcpy.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_int]
-    hip.hipMemcpy.restype = C.c_int
-    assert hip.hipMemcpy(out.data_ptr(), address, 4 * n, 3) == 0  # hipMemcpyDeviceToDevice
-    return out.cpu().numpy()
+    """n int32 from a raw device address on the host (the plan lives in memory torch does not own):
+    read through a tensor view of that address, by the runtime torch itself has loaded."""
+    return torch.as_tensor(_RawInts(address, n), device=DEV).clone().cpu().numpy()
 
 
 def one_job(spec, seed):
@@ -60,13 +63,31 @@ def one_job(spec, seed):
     ex1, em1 = torch.zeros_like(g["expert_x"]), torch.full_like(g["expert_meta"], -9)
     held = torch.cuda.memory_allocated(DEV)
     where = C.c_void_p()
-    rc = lib.moe_a2a_dispatch_recv_static(C.byref(a.shape), p(g["recv_buf"]), p(g["recv_meta"]),
-                                          p(g["recv_counts"]), R, cap, p(num1), p(ex1), p(em1),
-                                          C.byref(where), st)
-    assert rc == 0, lib.moe_a2a_strerror(rc)
-    assert where.value, "no plan address came back"
+
+    def call_static(stream):
+        rc = lib.moe_a2a_dispatch_recv_static(C.byref(a.shape), p(g["recv_buf"]), p(g["recv_meta"]),
+                                              p(g["recv_counts"]), R, cap, p(num1), p(ex1), p(em1),
+                                              C.byref(where), stream)
+        assert rc == 0, lib.moe_a2a_strerror(rc)
+        assert where.value, "no plan address came back"
+
+    call_static(st)  # (the first call on a GPU also looks the buffer's address up)
     assert torch.cuda.memory_allocated(DEV) == held > before  # torch's pool saw no allocation by the call
     torch.cuda.synchronize()
+    # The same call while the stream is being captured: a device allocation or free by anyone
+    # (hipMalloc, hipFree, torch's allocator) is refused during a capture and would fail it, so a
+    # capture that ends well shows that the call made none. The replay then has to do the work.
+    first_address = where.value
+    num1.fill_(-1); ex1.zero_(); em1.fill_(-9)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        call_static(C.c_void_p(torch.cuda.current_stream().cuda_stream))
+    assert where.value == first_address
+    assert bool((num1 == -1).all())  # captured, not run
+    graph.replay()
+    torch.cuda.synchronize()
+    del graph
 
     cnt = num0.cpu().numpy()
     assert np.array_equal(cnt, run_oracle(world)[1].expert_num_tokens)
