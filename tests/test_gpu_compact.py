@@ -63,6 +63,32 @@ def test_compact_layout_matches_the_oracle_and_the_padded_layout(name, plan):
         assert torch.equal(ys[r], ys_ref[r]), r
 
 
+def _edge_shapes():
+    from tests.test_gpu_parity import EDGE
+    return EDGE
+
+
+@pytest.mark.parametrize("name", sorted(_edge_shapes()))
+def test_compact_layout_on_the_edge_shapes(name):
+    """Rows that are not 16 bytes long, one local expert, 256 local experts (the prefix table in LDS
+    instead of registers), K = E, tiny and wide rows: `y` and the compact rows equal the oracle's."""
+    print(f"compact edge {name}", flush=True)
+    spec = dict(dict(routing="uniform", weights="rand"), **_edge_shapes()[name])
+    world = generate_world(spec, 31)
+    cfg, W = world[0][0], len(world)
+    dev = [d.to(DEV) for _, d, _, _ in world]
+    want = run_oracle(world)
+    for plan in (True, False):
+        lw = LocalWorld(cfg, W, device=DEV, layout="compact", reuse_placement=plan)
+        ys = lw.run(dev)
+        torch.cuda.synchronize()
+        for r in range(W):
+            R = int(want[r].expert_num_tokens.sum())
+            assert np.array_equal(bits(lw.trace[r]["expert_x"][:R]), want[r].expert_rows), (plan, r)
+            assert np.array_equal(lw.trace[r]["expert_meta"][:R].cpu().numpy(), want[r].expert_meta_rows), (plan, r)
+            assert np.array_equal(bits(ys[r]), want[r].y), (plan, r)
+
+
 @pytest.mark.parametrize("binding", ["ctypes", "ext"])
 def test_compact_layout_through_both_bindings(binding):
     world, cfg, dev = on_gpu("C3", 22)

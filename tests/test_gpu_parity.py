@@ -160,6 +160,11 @@ EDGE = {
                                           max_num_tokens=11, num_tokens="uniform", dtype="fp16"),
     "k_above_fast_list": dict(world_size=2, num_experts=160, experts_per_token=72, hidden_dim=64,
                               max_num_tokens=3, num_tokens="full", dtype="bf16"),
+    "k_above_the_weights_kept_in_lds": dict(world_size=2, num_experts=320, experts_per_token=136, hidden_dim=40,
+                                            max_num_tokens=2, num_tokens="full", dtype="fp16"),
+    "three_entries_per_token_wave_per_entry": dict(world_size=4, num_experts=12, experts_per_token=3,
+                                                   hidden_dim=7168, max_num_tokens=40, num_tokens="uniform",
+                                                   dtype="bf16"),
 }
 
 
