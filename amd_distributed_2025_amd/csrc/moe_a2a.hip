@@ -2785,7 +2785,7 @@ long long group_items(long long rows, const Geometry& g) {
 
 extern "C" {
 
-const char* moe_a2a_version(void) { return "moe_a2a 0.5 gfx950"; }
+const char* moe_a2a_version(void) { return "moe_a2a 0.6 gfx950"; }
 
 #ifndef MOE_A2A_BUILD_ID
 #define MOE_A2A_BUILD_ID "unknown"

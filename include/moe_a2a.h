@@ -66,7 +66,7 @@ typedef struct moe_a2a_shape {
 } moe_a2a_shape;
 
 /* Library version / build probe. Returns a static string such as
- * "moe_a2a 0.5 gfx950"; the number changes with the ABI. Never NULL. */
+ * "moe_a2a 0.6 gfx950"; the number changes with the ABI. Never NULL. */
 const char* moe_a2a_version(void);
 
 /* Identifies the sources this library was built from: the first 16 hex digits of
