@@ -459,19 +459,21 @@ __global__ __launch_bounds__(64 * ROWS) void dispatch_send_kernel(
 // [0, E): entry a precedes entry b exactly when its composite key is smaller.
 // The host uses this kernel when (W + 2) * S fits an int.
 
-// Entries of a token that are ranked in one pass over the keys and then stored (2, 4 or 8). Fewer
-// per pass means more passes over the same keys (they stay in registers) and more barriers, but the
-// first rows leave sooner and the ranking of the next entries runs while they drain; a compute
-// unit has nothing else to do meanwhile, because all its workgroups rank at the same time.
-// Measured at K = 8, H = 7168: the four path kernels together take 0.5 us less with 4 than with 8
-// and another 0.1 to 0.3 us less with 2.
-#ifndef MOE_A2A_FAN
-#define MOE_A2A_FAN 2
+// FAN: entries of a token that are ranked in one pass over the keys and then stored (2, 4 or 8).
+// Fewer per pass means more passes over the keys and more barriers, but the first rows leave sooner
+// and the ranking of the next entries runs while they drain; a compute unit has nothing else to
+// do meanwhile, because all its workgroups rank at the same time. That pays while a pass is short.
+// Measured at K = 8, H = 7168, the chain of four kernels (stage 1 alone in brackets), us, with
+// 2 / 4 / 8: S = 2048 entries 36.5 / 36.9 / 37.4; S = 4096 73.9 / 75.4 / 74.5 (15.7 / 14.2 / 15.2);
+// S = 8192 168.7 / 167.9 / 164.4 (31.6 / 31.8 / 29.0); S = 12288 233.2 / 230.5 / 222.6 (50.3 / 42.9 /
+// 38.8); S = 32768 693.6 / 615.0 / 567.7 (245.4 / 169.4 / 130.6). The host takes 2 up to
+// MOE_A2A_FAN2_MAX_ENTRIES entries and 8 above.
+#ifndef MOE_A2A_FAN2_MAX_ENTRIES
+#define MOE_A2A_FAN2_MAX_ENTRIES 4096
 #endif
-constexpr int FAN = MOE_A2A_FAN;
-static_assert(FAN == 2 || FAN == 4 || FAN == 8, "pairs of 16-bit counts, at most one DPP row of 16 lanes per pair");
+inline int fan_of(long long S) { return S <= MOE_A2A_FAN2_MAX_ENTRIES ? 2 : 8; }
 
-template <typename V, int NV>
+template <typename V, int NV, int FAN>
 __global__ __launch_bounds__(BLOCK) void dispatch_fanout_kernel(
     const V* __restrict__ x, const int* __restrict__ indices, int T, int K, int nle, int E, int W,
     uint32_t magic, int rank, int row_vecs, int chunks, V* __restrict__ send_buf,
@@ -575,7 +577,7 @@ __global__ __launch_bounds__(BLOCK) void dispatch_fanout_kernel(
 // the whole step 0.3 us shorter than with 256 lanes; 1024 lanes (one chunk per
 // row) 0.5 us longer.
 
-template <typename V, int BLK, int NV, bool POW2>
+template <typename V, int BLK, int NV, bool POW2, int FAN>
 __global__ __launch_bounds__(BLK) void dispatch_fanout_wide_kernel(
     const V* __restrict__ x, const int* __restrict__ indices, int T, int K, int nle, int E, int W,
     uint32_t magic, int nle_shift, int order_bits, int rank, int row_vecs, int chunks,
@@ -584,6 +586,7 @@ __global__ __launch_bounds__(BLK) void dispatch_fanout_wide_kernel(
   constexpr int NW = BLK / 64;
   constexpr int KEYS = SCAN_UNROLL * BLOCK / BLK;  // a batch stays SCAN_UNROLL * BLOCK keys
   constexpr int PAIRS = FAN / 2;
+  static_assert(FAN == 2 || FAN == 4 || FAN == 8, "pairs of 16-bit counts, one DPP row of 16 lanes per pair");
   static_assert(NW <= 16 && KEYS >= 1, "one DPP row of 16 lanes sums the waves");
   __shared__ int part[NW * PAIRS];
   __shared__ int total[PAIRS];
@@ -2828,6 +2831,7 @@ int moe_a2a_dispatch_send(const moe_a2a_shape* s, const void* x, const int32_t* 
   f.chunks = (f.row_vecs + BLOCK - 1) / BLOCK;
   if (s->experts_per_token >= MOE_A2A_FANOUT_MIN_K && (s->world_size + 2ll) * S <= INT_MAX &&
       items_fit(num_tokens, f.chunks)) {
+    const int fan = fan_of(S);
 #ifndef MOE_A2A_FANOUT_WIDE
 #define MOE_A2A_FANOUT_WIDE 1
 #endif
@@ -2844,31 +2848,43 @@ int moe_a2a_dispatch_send(const moe_a2a_shape* s, const void* x, const int32_t* 
       const bool pow2 = (g.nle & (g.nle - 1)) == 0;
       int nle_shift = 0;
       while ((1 << nle_shift) < g.nle) ++nle_shift;
-#define LAUNCH_W(V, NV, POW2)                                                                  \
-  dispatch_fanout_wide_kernel<V, WIDE, NV, POW2><<<wgrid, WIDE, 0, st>>>(                      \
+#define LAUNCH_W(V, NV, POW2, FAN)                                                             \
+  dispatch_fanout_wide_kernel<V, WIDE, NV, POW2, FAN><<<wgrid, WIDE, 0, st>>>(                 \
       (const V*)x, indices, num_tokens, s->experts_per_token, g.nle, s->num_experts,           \
       s->world_size, g.magic, nle_shift, order_bits, s->rank, f.row_vecs, wchunks,             \
       (V*)send_buf, send_meta, send_counts, send_slot)
+#define LAUNCH_WF(V, NV, POW2)                       \
+  do {                                               \
+    if (fan == 2) LAUNCH_W(V, NV, POW2, 2);          \
+    else LAUNCH_W(V, NV, POW2, 8);                   \
+  } while (0)
 #define LAUNCH_WV(V)                                                  \
   do {                                                                \
-    if (fnv == 2) { if (pow2) LAUNCH_W(V, 2, true); else LAUNCH_W(V, 2, false); } \
-    else { if (pow2) LAUNCH_W(V, 1, true); else LAUNCH_W(V, 1, false); }          \
+    if (fnv == 2) { if (pow2) LAUNCH_WF(V, 2, true); else LAUNCH_WF(V, 2, false); } \
+    else { if (pow2) LAUNCH_WF(V, 1, true); else LAUNCH_WF(V, 1, false); }          \
   } while (0)
       if (f.vec16) LAUNCH_WV(b128);
       else LAUNCH_WV(uint16_t);
 #undef LAUNCH_WV
+#undef LAUNCH_WF
 #undef LAUNCH_W
       return launch_status();
     }
     const int fgrid = s->world_size + mover_blocks((long long)num_tokens * f.chunks);
-#define LAUNCH(V)                                                                              \
-  dispatch_fanout_kernel<V, 1><<<fgrid, BLOCK, 0, st>>>(                                       \
+#define LAUNCH_F(V, FAN)                                                                       \
+  dispatch_fanout_kernel<V, 1, FAN><<<fgrid, BLOCK, 0, st>>>(                                  \
       (const V*)x, indices, num_tokens, s->experts_per_token, g.nle, s->num_experts,           \
       s->world_size, g.magic, s->rank, f.row_vecs, f.chunks, (V*)send_buf, send_meta,          \
       send_counts, send_slot)
+#define LAUNCH(V)                         \
+  do {                                    \
+    if (fan == 2) LAUNCH_F(V, 2);         \
+    else LAUNCH_F(V, 8);                  \
+  } while (0)
     if (f.vec16) LAUNCH(b128);  // one vector per lane is the only shape this kernel is launched with
     else LAUNCH(uint16_t);
 #undef LAUNCH
+#undef LAUNCH_F
     return launch_status();
   }
   const int grid = s->world_size + mover_blocks(group_items(S, g));
