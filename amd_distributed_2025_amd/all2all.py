@@ -480,41 +480,42 @@ class LocalWorld:
         self._sources = {}  # phase -> the source tables of the gathering exchange
         self.trace: List[dict] = [dict() for _ in range(world_size)]
 
-    def _exchange(self, phase: str, sent: List[Tuple[torch.Tensor, torch.Tensor, torch.Tensor]]):
-        W = self.world_size
+    def _exchange_hints(self, phase: str, sent):
+        """Host-side row counts [src][dst] that size the launches of one exchange, or None."""
         if self.exact_hints == "last":  # the counts read back by the previous run of the same job
-            host = self._last_counts[phase]
-        else:
-            host = torch.stack([s[0] for s in sent]).cpu().tolist() if self.exact_hints else None  # [src][dst]
-            self._last_counts[phase] = host
-        got = []
+            return self._last_counts[phase]
+        host = torch.stack([s[0] for s in sent]).cpu().tolist() if self.exact_hints else None
+        self._last_counts[phase] = host
+        return host
+
+    def _deliver(self, phase: str, r: int, sent, host):
+        """The inbound half of one exchange for rank r: (counts, buf, meta, rows or None)."""
+        W, dst = self.world_size, self.ranks[r]
+        rc, rb, rm = dst.inbound_buffers(phase)
+        # (with "last" the host counts are an earlier run's: they size launches and are no
+        # statement about this run)
+        total = sum(host[s][r] for s in range(W)) if host is not None else None
         if W <= GATHER_MAX_RANKS:
             # one launch per destination copies every source's segment and delivers the counts
             sources = self._sources.get(phase)
             if sources is None:  # (the workspaces the tables point into live as long as the ranks)
                 sources = self._sources[phase] = gather_sources(self.ranks, phase)
             loose = max(1, 2 * self.ranks[0].max_rows_out // W)
-            for r, dst in enumerate(self.ranks):
-                rc, rb, rm = dst.inbound_buffers(phase)
-                per_source = max(host[s][r] for s in range(W)) if host is not None else loose
-                exchange_gather(dst, sources, rc, rb, rm, min(per_source, rb.shape[0]))
-                # (with "last" these are an earlier run's counts: they size launches and are no
-                # statement about this run)
-                got.append((rc, rb, rm, sum(host[s][r] for s in range(W)) if host is not None else None))
-            return got
-        per_dst = torch.stack([s[0] for s in sent]).t().contiguous()  # [dst, src]
+            per_source = max(host[s][r] for s in range(W)) if host is not None else loose
+            exchange_gather(dst, sources, rc, rb, rm, min(per_source, rb.shape[0]))
+            return rc, rb, rm, total
+        rc.copy_(torch.stack([s[0][r] for s in sent]))
         bound = sent[0][1].shape[0]
-        for r, dst in enumerate(self.ranks):
-            rc, rb, rm = dst.inbound_buffers(phase)
-            rc.copy_(per_dst[r])
-            for s, src in enumerate(self.ranks):
-                hint = host[s][r] if host is not None else min(bound, sent[s][1].shape[0])
-                if host is not None and hint == 0 and self.exact_hints != "last":
-                    continue  # the counts were read back: this leg is known to be empty
-                exchange_leg(src, dst, sent[s][0], sent[s][1], sent[s][2], rc, rb, rm, max(hint, 1))
-            total = sum(host[s][r] for s in range(W)) if host is not None else None
-            got.append((rc, rb, rm, total))
-        return got
+        for s, src in enumerate(self.ranks):
+            hint = host[s][r] if host is not None else min(bound, sent[s][1].shape[0])
+            if host is not None and hint == 0 and self.exact_hints != "last":
+                continue  # the counts were read back: this leg is known to be empty
+            exchange_leg(src, dst, sent[s][0], sent[s][1], sent[s][2], rc, rb, rm, max(hint, 1))
+        return rc, rb, rm, total
+
+    def _exchange(self, phase: str, sent: List[Tuple[torch.Tensor, torch.Tensor, torch.Tensor]]):
+        host = self._exchange_hints(phase, sent)
+        return [self._deliver(phase, r, sent, host) for r in range(self.world_size)]
 
     def run(self, rank_data: Sequence[RankTestData], accumulate: bool = False,
             expert: Optional[Callable] = None) -> List[torch.Tensor]:
@@ -532,10 +533,10 @@ class LocalWorld:
             c, b, m, sl = a.dispatch_send(d.x, d.indices, want_slots=True)
             sent.append((c, b, m))
             self.trace[r].update(send_counts=c, send_buf=b, send_meta=m, send_slot=sl)
-        got = self._exchange("dispatch", sent)
+        host = self._exchange_hints("dispatch", sent)
         back = []
         for r, a in enumerate(self.ranks):
-            rc, rb, rm, total = got[r]
+            rc, rb, rm, total = self._deliver("dispatch", r, sent, host)
             num, ex, em = a.dispatch_recv(rc, rb, rm, total)
             ey = a.expert_scale(ex, num, total) if expert is None else expert(a, ex, num, total)
             bc, bb, bm = a.combine_send(em, ey, num, total)
@@ -543,11 +544,11 @@ class LocalWorld:
             self.trace[r].update(recv_counts=rc, recv_buf=rb, recv_meta=rm, expert_num_tokens=num,
                                  expert_x=ex, expert_meta=em, expert_y=ey,
                                  back_counts=bc, back_buf=bb, back_meta=bm)
-        got = self._exchange("combine", back)
+        host = self._exchange_hints("combine", back)
         ys = []
         for r, a in enumerate(self.ranks):
-            rc, rb, rm, _ = got[r]
             d = rank_data[r]
+            rc, rb, rm, _ = self._deliver("combine", r, back, host)
             if accumulate:
                 y = torch.zeros(cfg.max_num_tokens, cfg.hidden_dim, dtype=cfg.out_dtype, device=self.device)
             else:
