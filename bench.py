@@ -92,6 +92,8 @@ def parse_args():
                     help="how the host class reaches the C ABI: ctypes, or the torch extension built with load_inline")
     ap.add_argument("--no-extra-workloads", action="store_true",
                     help="skip the C5 block and the C4 block with the reference's input rules (fp16, rand weights)")
+    ap.add_argument("--no-entry-points", action="store_true",
+                    help="skip the timings of custom_kernel and of the class surface (they step every rank of the job)")
     return ap.parse_args()
 
 
@@ -412,7 +414,7 @@ def main():
 
     # (both entry-point sections make workspaces of their own for every rank of the job: they are for
     # the task's sizes and are left out for the larger row counts, and each frees what it made)
-    entry_points = args.workload in WORKLOADS
+    entry_points = args.workload in WORKLOADS and not args.no_entry_points
     world_dev = [(c, d, r, w) for (c, _, r, w), d in zip(world, data)]
     set_peer_inputs(world_dev)
 
