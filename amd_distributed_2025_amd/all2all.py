@@ -518,14 +518,18 @@ class LocalWorld:
         return [self._deliver(phase, r, sent, host) for r in range(self.world_size)]
 
     def run(self, rank_data: Sequence[RankTestData], accumulate: bool = False,
-            expert: Optional[Callable] = None) -> List[torch.Tensor]:
+            expert: Optional[Callable] = None, only: Optional[int] = None) -> List[torch.Tensor]:
         """`ref_kernel` (all2all/reference.py:256-272) for every rank; returns each
         rank's `y[:num_tokens]`. Intermediates are kept in `self.trace[r]`.
 
         `expert(rank_object, expert_x, expert_num_tokens, rows_hint)` returns the rank's
         `expert_y [nle, max_recv, hidden_dim]` of `out_dtype`: what a model runs where the
         reference has `expert_x.to(out_dtype) * (1 + rank)` (reference.py:262), for example layers
-        of `HIPAllToAll.expert_gemm`. None is the reference's stand-in."""
+        of `HIPAllToAll.expert_gemm`. None is the reference's stand-in.
+
+        `only=r`: the caller wants rank r's result alone. Every rank still dispatches, runs its
+        experts and sends back (rank r's rows come from all of them), but the return exchange and
+        the weighted sum run for rank r only; the other entries of the result are None."""
         cfg = self.cfg
         sent = []
         for r, a in enumerate(self.ranks):
@@ -547,6 +551,9 @@ class LocalWorld:
         host = self._exchange_hints("combine", back)
         ys = []
         for r, a in enumerate(self.ranks):
+            if only is not None and r != only:
+                ys.append(None)
+                continue
             d = rank_data[r]
             rc, rb, rm, _ = self._deliver("combine", r, back, host)
             if accumulate:

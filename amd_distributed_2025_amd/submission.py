@@ -12,7 +12,9 @@ With `world_size == 1` nothing has to be registered.
 A harness calls the entry point again and again on jobs of one shape. The first
 call of a job (a shape and the token counts of its ranks) runs launch by launch
 and reads the exchanged counts back to size its launches; from the second call
-on the job is a HIP graph captured once: the inputs are copied into buffers the
+on the job is a HIP graph captured once (one per rank asked for: a call needs
+every rank's dispatch, experts and send-back, but only the caller's return
+exchange and weighted sum): the inputs are copied into buffers the
 graph reads, the graph is replayed, the result is copied out. The graph's
 launches are sized by the counts of the first call; sizes are a matter of speed
 only, every kernel moves what the device-side counts of the call at hand say.
@@ -28,7 +30,7 @@ from .task import MoEConfig, RankTestData, input_t, output_t
 
 _peers: Optional[Sequence[input_t]] = None
 _worlds: Dict[Tuple, "_World"] = {}
-MAX_CAPTURED_JOBS = 4  # graphs kept per job shape (each holds only launches; the buffers are the world's)
+MAX_CAPTURED_JOBS = 18  # graphs kept per job shape (each holds only launches; the buffers are the world's)
 
 
 def set_peer_inputs(inputs: Optional[Sequence[input_t]]) -> None:
@@ -48,7 +50,7 @@ class _World:
         self.indices = [torch.empty(T, K, dtype=torch.int32, device=device) for _ in range(world_size)]
         self.weights = [torch.empty(T, K, dtype=torch.float32, device=device) for _ in range(world_size)]
         self.seen: Dict[Tuple[int, ...], int] = {}
-        self.graphs: Dict[Tuple[int, ...], Tuple[torch.cuda.CUDAGraph, List[torch.Tensor]]] = {}
+        self.graphs: Dict[Tuple, Tuple[torch.cuda.CUDAGraph, List[torch.Tensor]]] = {}
 
     def _staged(self, tokens: Tuple[int, ...]) -> List[RankTestData]:
         """Views of the input buffers cut to the job's token counts, as rank inputs."""
@@ -60,30 +62,33 @@ class _World:
             out.append(d)
         return out
 
-    def run(self, everyone: Sequence[RankTestData]) -> List[torch.Tensor]:
+    def run(self, everyone: Sequence[RankTestData], only: Optional[int] = None) -> List[torch.Tensor]:
+        """One step of the job; `only=r` leaves out what only the other ranks' results need (their
+        return exchange and weighted sum) and returns None in their places."""
         tokens = tuple(int(d.num_tokens) for d in everyone)
         calls = self.seen.get(tokens, 0)
         self.seen[tokens] = calls + 1
         if calls == 0:  # launch by launch, reading the counts back: they size the later launches
             self.lw.exact_hints = True
-            return self.lw.run(everyone)
+            return self.lw.run(everyone, only=only)
         staged = self._staged(tokens)
         torch._foreach_copy_([d.x for d in staged] + [d.indices for d in staged] + [d.weights for d in staged],
                              [d.x for d in everyone] + [d.indices for d in everyone] + [d.weights for d in everyone])
-        if tokens not in self.graphs:
+        key = (tokens, only)
+        if key not in self.graphs:
             while len(self.graphs) >= MAX_CAPTURED_JOBS:
                 self.graphs.pop(next(iter(self.graphs)))
             # the counts sizing the launches are those the latest launch-by-launch run of this world
             # read back; a job of other token counts came in between only if it ran that way too
             self.lw.exact_hints = True
-            self.lw.run(staged)  # (also leaves every workspace buffer allocated before the capture)
+            self.lw.run(staged, only=only)  # (also leaves every workspace buffer allocated before the capture)
             self.lw.exact_hints = "last"
             torch.cuda.synchronize(self.lw.device)
             graph = torch.cuda.CUDAGraph()
             with torch.cuda.graph(graph):
-                ys = self.lw.run(staged)
-            self.graphs[tokens] = (graph, ys)
-        graph, ys = self.graphs[tokens]
+                ys = self.lw.run(staged, only=only)
+            self.graphs[key] = (graph, ys)
+        graph, ys = self.graphs[key]
         graph.replay()
         return ys
 
@@ -126,5 +131,5 @@ def custom_kernel(data: input_t) -> output_t:
             )
         everyone = [rank_data if r == rank else _peers[r][1].to(device) for r in range(world_size)]
     with torch.cuda.device(device):
-        ys = _world_for(cfg, world_size, device).run(everyone)
+        ys = _world_for(cfg, world_size, device).run(everyone, only=rank)
         return ys[rank].clone()

@@ -389,5 +389,10 @@ def test_custom_kernel_call_after_call_with_changing_inputs():
         want = run_oracle(world)
         for r in range(len(world)):
             assert np.array_equal(bits(ys[r]), want[r].y), f"zipf rank {r}"
+        # every rank in turn asks for its own rows (a captured job per rank asked for), twice over
+        for _ in range(2):
+            for r in range(len(world)):
+                y = custom_kernel(on_dev[r])
+                assert np.array_equal(bits(y), want[r].y), f"rank {r} alone"
     finally:
         set_peer_inputs(None)
