@@ -274,3 +274,17 @@ def test_a_pair_that_arrives_twice_is_added_twice_only_when_the_caller_says_pair
     one_of = [orc.combine_recv(bits(rows)[k], meta[k], weights.numpy(), T, "bf16") for k in (keep_first, keep_last)]
     assert any(np.array_equal(bits(y), w) for w in one_of)
     assert not np.array_equal(bits(y), both)
+
+
+@pytest.mark.parametrize("hidden_dim,tokens", [(2304, 640), (4608, 520), (7168, 513), (1024, 800)])
+def test_stage_one_above_4096_entries_with_long_rows(hidden_dim, tokens):
+    """Above 4096 entries per rank stage 1 ranks all of a token's entries in one pass over the keys
+    (two at a time below): rows of more than 256, more than 512 and of at most 256 vectors take the
+    three shapes of that kernel. Every buffer and `y` against the oracle, both kinds of receive half."""
+    print(f"stage 1, {tokens * 8} entries of {hidden_dim} elements", flush=True)
+    spec = dict(world_size=2, num_experts=16, experts_per_token=8, hidden_dim=hidden_dim,
+                max_num_tokens=tokens, num_tokens="full", routing="uniform", weights="softmax", dtype="bf16")
+    assert tokens * 8 > 4096
+    world = generate_world(spec, 31)
+    run_long(world, long_stream_rows=None)
+    run_long(world, long_stream_rows=0)
