@@ -150,13 +150,13 @@ def main():
     if args.weights:
         wl["weights"] = args.weights
 
-    def set_up(workload):
+    def set_up(workload, **layout):
         """The whole job once, so that every rank's inbound buffers hold the peers' segments."""
         world_ = generate_world(workload, args.seed)
         cfg_ = world_[0][0]
         data_ = [d.to(dev) for _, d, _, _ in world_]
         lw_ = LocalWorld(cfg_, len(world_), device=dev, reuse_placement=not args.no_placement_plan,
-                         long_stream_rows=args.long_stream_rows, binding=args.binding)
+                         long_stream_rows=args.long_stream_rows, binding=args.binding, **layout)
         ys_ = [y.clone() for y in lw_.run(data_)]
         torch.cuda.synchronize()
         return world_, cfg_, data_, lw_, ys_
@@ -374,8 +374,8 @@ def main():
     # rank 0 and the ranks that receive the most and the fewest rows, with their realised row
     # counts) and on C4 with the reference's own input rules (fp16 tokens and `rand` weights,
     # all2all/reference.py:16-17,37-43). One job each, set up like the main one.
-    def hot_path_of(workload, pick_ranks):
-        world_, cfg_, data_, lw_, _ = set_up(workload)
+    def hot_path_of(workload, pick_ranks, **layout):
+        world_, cfg_, data_, lw_, _ = set_up(workload, **layout)
         W_ = len(world_)
         rows = [int(lw_.trace[r]["recv_counts"].sum().item()) for r in range(W_)]
         res = {}
@@ -388,6 +388,8 @@ def main():
             res[str(r)] = {"rows_sent": T_r * cfg_.experts_per_token, "rows_received": R_r,
                            "hot_path_us": round(hot_r, 3), "hot_path_alg_bytes": alg_r,
                            "frac": round(alg_r / hot_r * 1e-3 / HBM_PEAK_GBPS, 4)}
+            if layout:
+                res[str(r)]["workspace_bytes"] = lw_.ranks[r].workspace_bytes()
         del lw_, data_
         torch.cuda.empty_cache()
         return res, rows
@@ -406,6 +408,12 @@ def main():
         out["c4_fp16_rand"] = dict(res[str(r0)], workload=f"C4 with dtype=fp16, weights=rand (the reference's "
                                    f"input rules), rank {r0}, seed={args.seed}",
                                    hot_path_frac_of_hbm_peak=res[str(r0)]["frac"])
+        # the same job with the expert-major buffers in the compact layout (rows of an expert at its
+        # offset, room for 2560 rows instead of 32 x 2048): the same four stages, a twentieth of the memory
+        res, _ = hot_path_of(WORKLOADS["C4"], lambda n: [r0], layout="compact", compact_rows=2560)
+        out["c4_compact_layout"] = dict(res[str(r0)], compact_rows=2560,
+                                        workspace_bytes_padded_layout=lw.ranks[r0].workspace_bytes(),
+                                        hot_path_frac_of_hbm_peak=res[str(r0)]["frac"])
 
     # ---- the reference's entry point: one call steps the whole job on this GPU (all ranks' kernels and
     # one gathering exchange launch per rank and direction). The first call of a job runs launch by
