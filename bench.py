@@ -370,7 +370,7 @@ def main():
         out["hot_path_frac_min_over_ranks"] = min(fr)
         out["hot_path_frac_mean_over_ranks"] = round(sum(fr) / len(fr), 4)
 
-    # ---- the same path on the other workload BASELINE names at this shape (C5: Zipf-skewed routing;
+    # ---- the same path on the skewed workload of this shape (C5: Zipf-skewed routing;
     # rank 0 and the ranks that receive the most and the fewest rows, with their realised row
     # counts) and on C4 with the reference's own input rules (fp16 tokens and `rand` weights,
     # all2all/reference.py:16-17,37-43). One job each, set up like the main one.
