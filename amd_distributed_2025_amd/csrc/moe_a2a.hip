@@ -155,6 +155,14 @@ __device__ __forceinline__ int first_use(int v) {
   return v;
 }
 
+// A float32 value that counts as computed and rounded at this point: the compiler may not fuse the
+// multiplication that made it with the conversion that follows. (Fused, a product rounded to fp16
+// becomes v_fma_mixlo_f16 with an addend of +0, and -0 * scale + 0 is +0 where the product is -0.)
+__device__ __forceinline__ float rounded_here(float v) {
+  asm volatile("" : "+v"(v));
+  return v;
+}
+
 // Loads through a pointer that went through unknown_origin() and were issued before issued_here()
 // stay before it. The compiler otherwise sinks a load whose value is only used under a condition
 // into that condition's block, behind whatever the condition waits for; an asm statement that
@@ -1753,8 +1761,9 @@ __global__ __launch_bounds__(BLOCK) void expert_scale_kernel(
         const uint32_t w = get_word(v, e);
         // .to(out_dtype), then times (1 + rank) in float32, rounded once
         const uint32_t o = Pair16<DOUT>::round(Pair16<DIN>::lo(w), Pair16<DIN>::hi(w));
-        h[e] = Pair16<DOUT>::canonical(Pair16<DOUT>::round(__fmul_rn(Pair16<DOUT>::lo(o), scale),
-                                                           __fmul_rn(Pair16<DOUT>::hi(o), scale)));
+        const float lo = rounded_here(__fmul_rn(Pair16<DOUT>::lo(o), scale));
+        const float hi = rounded_here(__fmul_rn(Pair16<DOUT>::hi(o), scale));
+        h[e] = Pair16<DOUT>::canonical(Pair16<DOUT>::round(lo, hi));
       }
       return from_words<V>(h);
     });
@@ -1789,8 +1798,9 @@ __global__ __launch_bounds__(64 * ROWS) void expert_scale_wave_kernel(
         const uint32_t w = p.v[j][e];
         // .to(out_dtype), then times (1 + rank) in float32, rounded once
         const uint32_t o = Pair16<DOUT>::round(Pair16<DIN>::lo(w), Pair16<DIN>::hi(w));
-        h[e] = Pair16<DOUT>::canonical(Pair16<DOUT>::round(__fmul_rn(Pair16<DOUT>::lo(o), scale),
-                                                           __fmul_rn(Pair16<DOUT>::hi(o), scale)));
+        const float lo = rounded_here(__fmul_rn(Pair16<DOUT>::lo(o), scale));
+        const float hi = rounded_here(__fmul_rn(Pair16<DOUT>::hi(o), scale));
+        h[e] = Pair16<DOUT>::canonical(Pair16<DOUT>::round(lo, hi));
       }
       p.v[j] = from_words<b128>(h);
     }

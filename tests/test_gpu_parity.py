@@ -308,6 +308,71 @@ def test_rounding_of_every_bit_pattern_through_combine_and_expert(name):
     assert np.isnan(orc.b16_to_f32(got[nan], name)).all()
 
 
+def every_pattern(H):
+    """All 65536 bit patterns laid into rows of H elements (the last row wraps around)."""
+    rows = -(-65536 // H)
+    return (np.arange(rows * H, dtype=np.uint32) % 65536).astype(np.uint16).reshape(rows, H)
+
+
+@pytest.mark.parametrize("name_in,name_out", [("bf16", "bf16"), ("fp16", "fp16"), ("fp16", "bf16"), ("bf16", "fp16")])
+@pytest.mark.parametrize("H,nle", [(100, 1), (2048, 65), (520, 3)])
+def test_expert_standin_on_every_bit_pattern_through_every_kernel(name_in, name_out, H, nle):
+    """The simulated expert has three kernels: rows that are not a multiple of 16 bytes move element by
+    element (H = 100), more than 64 local experts take a workgroup per row (nle = 65), the rest a wave
+    per row. Every bit pattern, negative zero among them, times 1 (rank 0) and times 3, in every
+    pairing of the two types, against the oracle."""
+    print(f"expert stand-in, all patterns: {name_in}->{name_out} H={H} nle={nle}", flush=True)
+    pats = every_pattern(H)
+    rows = pats.shape[0]
+    for rank, W in ((0, 1), (2, 3)):
+        cfg = MoEConfig(W * nle, 1, H, rows, DTYPES[name_in], DTYPES[name_out])
+        a = LocalWorld(cfg, W, device=DEV).ranks[rank]
+        ex = torch.zeros(nle, rows * W, H, dtype=DTYPES[name_in], device=DEV)
+        ex[nle - 1, :rows] = from_bits(pats, DTYPES[name_in]).to(DEV)
+        counts = torch.zeros(nle, dtype=torch.int32, device=DEV)
+        counts[nle - 1] = rows
+        ey = a.expert_scale(ex, counts, rows)
+        torch.cuda.synchronize()
+        want = orc.expert_scale(pats, rank, name_in, name_out)
+        got = bits(ey[nle - 1, :rows])
+        nan = np.isnan(orc.b16_to_f32(want, name_out))
+        assert np.array_equal(got[~nan], want[~nan]), f"scale {1 + rank}"
+        assert np.isnan(orc.b16_to_f32(got[nan], name_out)).all()
+        zero_in = (pats & 0x7FFF) == 0
+        assert np.array_equal(got[zero_in], pats[zero_in]), "a zero keeps its sign"
+
+
+@pytest.mark.parametrize("name", ["bf16", "fp16"])
+def test_combine_on_every_bit_pattern_on_rows_moved_element_by_element(name):
+    """The weighted sum on rows that are not a multiple of 16 bytes (H = 100): every bit pattern as
+    first addend, a random second one, weights that force roundings."""
+    dt = DTYPES[name]
+    H, K = 100, 2
+    pats = every_pattern(H)
+    T = pats.shape[0]
+    rng = np.random.default_rng(4)
+    second = orc.f32_to_b16(rng.standard_normal((T, H)).astype(np.float32) * 3, name)
+    cfg = MoEConfig(2, K, H, T, dt, dt)
+    a = LocalWorld(cfg, 1, device=DEV).ranks[0]
+    ret_buf = torch.cat([from_bits(pats, dt), from_bits(second, dt)]).to(DEV)
+    meta = np.zeros((2 * T, 5), np.int32)
+    meta[:T, 2] = np.arange(T); meta[T:, 2] = np.arange(T); meta[T:, 3] = 1
+    w = (1 + rng.random((T, K), dtype=np.float32) * 2.0 ** -6).astype(np.float32)
+    w[::4, 0] = 1.0
+    counts = torch.tensor([2 * T], dtype=torch.int32, device=DEV)
+    y = torch.empty(T, H, dtype=dt, device=DEV)
+    a.combine_recv(y, torch.from_numpy(w).to(DEV), counts, ret_buf, torch.from_numpy(meta).to(DEV),
+                   accumulate=False)
+    torch.cuda.synchronize()
+    want = orc.combine_recv(np.concatenate([pats, second]), meta, w, T, name)
+    got = bits(y)
+    nan = np.isnan(orc.b16_to_f32(want, name))
+    assert np.array_equal(got[~nan], want[~nan])
+    assert np.isnan(orc.b16_to_f32(got[nan], name)).all()
+    if name == "bf16":
+        assert (got[nan] == 0x7FC0).all()
+
+
 def test_custom_kernel_drop_in():
     """`custom_kernel(data)` with the reference's tuple, checked the way the
     reference's check_implementation does (allclose rtol 1e-2, atol 5e-3,
