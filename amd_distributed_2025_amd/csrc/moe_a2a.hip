@@ -365,6 +365,16 @@ struct RowsScan {
       consume(test, cnt);
     }
   }
+  // Adds the counts over keys [from, to): keys past the n_load the scan began with, readable now
+  // that the caller knows the stream is that long (a stream longer than the hint it was launched with).
+  template <typename Test>
+  __device__ __forceinline__ void extend(const Keys& keys, int from, int to, Test test, int (&cnt)[ROWS]) {
+    n = to;
+    for (b = from; b < to; b += SCAN_UNROLL * STEP) {
+      issue(keys);
+      consume(test, cnt);
+    }
+  }
 };
 
 // Total of cnt[wave] over the workgroup, returned to the lanes of that wave:
@@ -1065,11 +1075,17 @@ __global__ __launch_bounds__(64 * ROWS) void dispatch_recv_kernel(
 #pragma unroll
     for (int r = 0; r < ROWS; ++r) rle[r] = floormod(re[r], nle, magic);
     int cnt[ROWS];
-    scan.finish(key, COMPACT ? R : min(i0 + ROWS - 1, R), [&](int r, int e2, int i2) {
+    auto precedes = [&](int r, int e2, int i2) {
       const int le2 = floormod(e2, nle, magic);
       if constexpr (COMPACT) return (le2 < rle[r]) | ((le2 == rle[r]) & (i2 < i0 + r));
       else return (le2 == rle[r]) & (i2 < i0 + r);
-    }, cnt);
+    };
+    scan.finish(key, COMPACT ? R : min(i0 + ROWS - 1, R), precedes, cnt);
+    if constexpr (COMPACT) {
+      // the scan began with the `limit` keys that were known to be readable; a stream longer than
+      // that (a hint below the row count) has rows of lower experts behind them as well
+      if (R > limit) scan.extend(key, limit, R, precedes, cnt);
+    }
     const int pos = rows_reduce(cnt, part, parity++, wave, lane);
 
     if (i < R && pos < max_recv) {

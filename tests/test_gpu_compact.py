@@ -226,3 +226,64 @@ def test_compact_workspace_at_c4_is_a_fraction_of_the_padded_one():
           f"whole workspace of a rank {a.workspace_bytes() / 1e6:.1f} MB", flush=True)
     assert expert_bytes < 100e6 and padded_bytes > 1.8e9
     assert a.workspace_bytes() < 250e6
+
+
+@pytest.mark.parametrize("layout", ["compact", "padded"])
+@pytest.mark.parametrize("factor", [0.0, 0.05, 0.4, 1.5])
+def test_launch_sizes_below_and_above_the_row_counts(layout, factor):
+    """`rows_hint` only sizes launches: every half must move the whole stream when the hint is far
+    below the rows that arrive (and when it is above). The row counts that size the launches of a
+    skewed job are scaled by `factor` before they reach the halves."""
+    print(f"hints x {factor}, {layout}", flush=True)
+    spec = dict(world_size=4, num_experts=32, experts_per_token=6, hidden_dim=24, max_num_tokens=95,
+                num_tokens="full", routing="zipf", weights="rand", dtype="bf16")
+    world = generate_world(spec, 90003)
+    cfg, W = world[0][0], 4
+    dev = [d.to(DEV) for _, d, _, _ in world]
+    want = run_oracle(world)
+    for plan in (True, False):
+        lw = LocalWorld(cfg, W, device=DEV, layout=layout, reuse_placement=plan)
+        counts_of = lw._exchange_hints
+        lw._exchange_hints = lambda phase, sent: [[int(c * factor) for c in row] for row in counts_of(phase, sent)]
+        ys = lw.run(dev)
+        torch.cuda.synchronize()
+        for r in range(W):
+            g, n = lw.trace[r], int(want[r].expert_num_tokens.sum())
+            assert np.array_equal(g["expert_num_tokens"].cpu().numpy(), want[r].expert_num_tokens), r
+            if layout == "compact":
+                assert np.array_equal(bits(g["expert_x"][:n]), want[r].expert_rows), r
+                assert np.array_equal(g["expert_meta"][:n].cpu().numpy(), want[r].expert_meta_rows), r
+                assert np.array_equal(bits(g["expert_y"][:n]), want[r].expert_y_rows), r
+            assert np.array_equal(bits(g["back_buf"][:n]), want[r].back_buf), r
+            assert np.array_equal(bits(ys[r]), want[r].y), r
+
+
+@pytest.mark.parametrize("binding", ["ctypes", "ext"])
+def test_class_surface_in_the_compact_layout_on_a_skewed_job(binding):
+    """`dispatch()` / `combine()` without row counts on the host size their launches for the rows a
+    rank sends; with skewed routing some ranks receive more than that (here 749 and 654 rows for
+    570 sent)."""
+    from amd_distributed_2025_amd import run_lockstep
+
+    spec = dict(world_size=4, num_experts=32, experts_per_token=6, hidden_dim=24, max_num_tokens=95,
+                num_tokens="full", routing="zipf", weights="rand", dtype="bf16")
+    world = generate_world(spec, 90003)
+    cfg, W = world[0][0], 4
+    dev = [d.to(DEV) for _, d, _, _ in world]
+    want = run_oracle(world)
+    assert max(int(t.recv_counts.sum()) for t in want) > cfg.max_num_tokens * cfg.experts_per_token
+
+    def rank_main(rank, exchange):
+        ata = HIPAllToAll(cfg, rank, W, exchange=exchange, device=DEV, binding=binding, layout="compact")
+        num, ex, em = ata.dispatch(dev[rank].x, dev[rank].indices)
+        ey = ata.expert_scale(ex, num)
+        y = torch.zeros(cfg.max_num_tokens, cfg.hidden_dim, dtype=cfg.out_dtype, device=DEV)
+        ata.combine(y, dev[rank].weights, em, ey, num)
+        torch.cuda.synchronize()
+        return y[: dev[rank].num_tokens].clone(), ex.clone(), em.clone()
+
+    for r, (y, ex, em) in enumerate(run_lockstep(W, rank_main, exact_hints=False, device=DEV)):
+        n = int(want[r].expert_num_tokens.sum())
+        assert np.array_equal(bits(ex[:n]), want[r].expert_rows), r
+        assert np.array_equal(em[:n].cpu().numpy(), want[r].expert_meta_rows), r
+        assert np.array_equal(bits(y), want[r].y), r
