@@ -165,6 +165,11 @@ EDGE = {
     "three_entries_per_token_wave_per_entry": dict(world_size=4, num_experts=12, experts_per_token=3,
                                                    hidden_dim=7168, max_num_tokens=40, num_tokens="uniform",
                                                    dtype="bf16"),
+    # more ranks than a wave has lanes: the per-rank vectors no longer fit one register per lane
+    "sixty_five_ranks": dict(world_size=65, num_experts=130, experts_per_token=5, hidden_dim=72,
+                             max_num_tokens=9, num_tokens="uniform", routing="zipf", dtype="bf16"),
+    "one_hundred_and_thirty_ranks": dict(world_size=130, num_experts=130, experts_per_token=4, hidden_dim=100,
+                                         max_num_tokens=7, num_tokens="full", dtype="fp16"),
 }
 
 
