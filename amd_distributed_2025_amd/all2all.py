@@ -41,7 +41,15 @@ META_DIM = 5
 LONG_STREAM_ROWS = {"dispatch": 8192, "combine": 4096}
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def _stream(device) -> int:
+    """The current HIP stream of `device` as an integer handle. The raw accessor costs a fraction of
+    a microsecond; `torch.cuda.current_stream()` builds a Stream object (about 5 us, a third of what
+    the host spends on a launch here)."""
+    if _raw_stream is not None and device.index is not None:
+        return _raw_stream(device.index)
     return torch.cuda.current_stream(device).cuda_stream
 
 

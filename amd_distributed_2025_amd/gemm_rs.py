@@ -18,6 +18,7 @@ from typing import List, Optional, Sequence, Tuple
 import torch
 
 from . import _binding
+from .all2all import _stream
 
 input_t = Tuple[torch.Tensor, torch.Tensor, Optional[torch.Tensor]]
 
@@ -69,7 +70,7 @@ def local_product(data: input_t, out: Optional[torch.Tensor] = None, binding: st
         out = torch.empty((m, n), dtype=inp.dtype, device=inp.device)
     elif tuple(out.shape) != (m, n) or out.dtype != inp.dtype or out.device != inp.device or not out.is_contiguous():
         raise ValueError(f"out must be a contiguous [{m}, {n}] {inp.dtype} tensor on {inp.device}")
-    stream = torch.cuda.current_stream(inp.device).cuda_stream
+    stream = _stream(inp.device)
     _binding.get(binding).linear(inp, weight, bias, out, stream)
     return out
 

@@ -485,6 +485,39 @@ def main():
             surf[b_name] = {"job_wall_us": round(us, 1), "per_rank_us": round(us / W, 1), "matches_step": same}
         out["class_surface_eager"] = dict(surf, measure="dispatch() + expert stand-in + combine() of every rank, one "
                                           "thread per rank, loose launch sizes, median wall time of 5 jobs")
+        # The threads of that job spend most of their time meeting each other (eight Python threads at
+        # four barriers); what the calls of ONE rank cost its process is seen on a job of a single rank
+        # with the rank's share of the shape (its local experts, the same tokens, rows and row length):
+        # time until the last launch is issued, and until the GPU has finished.
+        from amd_distributed_2025_amd.task import MoEConfig, RankTestData
+        solo_cfg = MoEConfig(cfg.num_experts // W, min(K, cfg.num_experts // W), H, cfg.max_num_tokens,
+                             cfg.in_dtype, cfg.out_dtype)
+        d0 = data[r0]
+        solo_idx = (d0.indices % solo_cfg.num_experts)[:, : solo_cfg.experts_per_token].contiguous()
+        solo_w = d0.weights[:, : solo_cfg.experts_per_token].contiguous()
+        solo = {}
+        for b_name in ("ctypes", "ext"):
+            a1 = HIPAllToAll(solo_cfg, 0, 1, device=dev, binding=b_name)
+            y1 = torch.zeros(solo_cfg.max_num_tokens, H, dtype=cfg.out_dtype, device=dev)
+            issued, done = [], []
+            for i in range(25):
+                torch.cuda.synchronize()
+                t0 = time.perf_counter()
+                num, ex, em = a1.dispatch(d0.x, solo_idx)
+                ey = a1.expert_scale(ex, num)
+                a1.combine(y1, solo_w, em, ey, num)
+                t1 = time.perf_counter()
+                torch.cuda.synchronize()
+                t2 = time.perf_counter()
+                if i >= 5:
+                    issued.append((t1 - t0) * 1e6)
+                    done.append((t2 - t0) * 1e6)
+            solo[b_name] = {"issue_us": round(statistics.median(issued), 1), "wall_us": round(statistics.median(done), 1)}
+            del a1, y1
+            torch.cuda.empty_cache()
+        out["class_surface_eager"]["one_rank_job"] = dict(
+            solo, measure="dispatch() + stand-in + combine() on a job of one rank with this rank's share of the shape "
+                          "(no exchange, no other thread): host time to issue the launches, and wall time with the GPU's work")
 
     # ---- the expert computation a model runs between the two halves: the grouped GEMM over this
     # rank's expert-major rows (random weights; the stand-in of the reference stays in the step above)
